@@ -40,13 +40,15 @@ class CacheGroupSpec:
     head_dim: int
     window: int = 0  # 0: every earlier key stays visible
     value_dim: int = 0  # head size of the values where it differs from the keys' (0: the same)
+    # True: values are read from the key rows; the group keeps one pool and hands it out as both
+    values_in_keys: bool = False
 
     @property
     def value_head_dim(self) -> int:
         return self.value_dim or self.head_dim
 
     def geometry(self):
-        return (self.kv_heads, self.head_dim, self.window, self.value_head_dim)
+        return (self.kv_heads, self.head_dim, self.window, self.value_head_dim, self.values_in_keys)
 
 
 @dataclass(frozen=True)
@@ -160,8 +162,11 @@ class CacheManager:
             if allocate_pools:
                 shape = (len(group.entries), pool.num_pages, group.kv_heads, page_size)
                 self.key_pools.append(torch.empty(shape + (group.head_dim,), dtype=dtype, device=self.device))
-                self.value_pools.append(torch.empty(shape + (group.value_head_dim,), dtype=dtype,
-                                                    device=self.device))
+                if group.values_in_keys:
+                    self.value_pools.append(self.key_pools[-1])
+                else:
+                    self.value_pools.append(torch.empty(shape + (group.value_head_dim,), dtype=dtype,
+                                                        device=self.device))
             else:
                 self.key_pools.append(None)
                 self.value_pools.append(None)
@@ -187,8 +192,8 @@ class CacheManager:
         group = self.groups[group_index]
         element = torch.empty(0, dtype=self.dtype).element_size()
         # src/model/kv_manager.py:55-58
-        return (len(group.entries) * group.kv_heads * self.page_size
-                * (group.head_dim + group.value_head_dim) * element)
+        per_key = group.head_dim + (0 if group.values_in_keys else group.value_head_dim)
+        return len(group.entries) * group.kv_heads * self.page_size * per_key * element
 
     def pages_for_length(self, group_index: int, length: int, longest_step: Optional[int] = None) -> int:
         """Most pages that one request of ``length`` tokens holds in a group at any

@@ -118,6 +118,8 @@ class ModelSpec:
     # rows of a table ``[pass_rows, width]`` of vectors that calls of the run order may add to the
     # stream before they run (``LayerCall.enter``); 0: the model has none
     pass_rows: int = 0
+    # a norm of the embedded rows before the first block (its result is the residual stream)
+    embedding_norm: Optional[PartSpec] = None
 
     def __post_init__(self):
         if not self.blocks:

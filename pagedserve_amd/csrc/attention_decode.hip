@@ -197,10 +197,10 @@ extern "C" int ps_attention_decode_static(const void* q, int64_t q_stride, const
   if (dtype == PS_F32)
     return launch_decode<float>(q, q_stride, k_pool, v_pool, out, out_stride, partial, tok_list,
                                 tok_item, tok_pos, tables, table_width, count, heads, kv_heads,
-                                head_dim, page_size, num_pages, scale, window, splits, waves, AttnExtras{nullptr, nullptr, 0}, s);
+                                head_dim, page_size, num_pages, scale, window, splits, waves, AttnExtras{nullptr, nullptr, 0, 0.f}, s);
   return launch_decode<bf16_t>(q, q_stride, k_pool, v_pool, out, out_stride, partial, tok_list,
                                tok_item, tok_pos, tables, table_width, count, heads, kv_heads,
-                               head_dim, page_size, num_pages, scale, window, splits, waves, AttnExtras{nullptr, nullptr, 0}, s);
+                               head_dim, page_size, num_pages, scale, window, splits, waves, AttnExtras{nullptr, nullptr, 0, 0.f}, s);
 }
 
 // The partial records only (see pagedserve_hip.h).
@@ -211,7 +211,8 @@ extern "C" int ps_attention_decode_partial(const void* q, int64_t q_stride, cons
                                            const int* tables, int table_width, int count,
                                            int heads, int kv_heads, int head_dim, int page_size,
                                            int num_pages, float scale, int window, int splits,
-                                           int waves, const float* sink, int dtype, void* stream) {
+                                           int waves, const float* sink, float softcap, int dtype,
+                                           void* stream) {
   if (check_decode_sizes("ps_attention_decode_partial", count, heads, kv_heads, head_dim,
                          page_size, num_pages, table_width, window, splits, waves, dtype))
     return 1;
@@ -223,10 +224,10 @@ extern "C" int ps_attention_decode_partial(const void* q, int64_t q_stride, cons
   if (dtype == PS_F32)
     return launch_decode<float>(q, q_stride, k_pool, v_pool, nullptr, 0, partial, tok_list,
                                 tok_item, tok_pos, tables, table_width, count, heads, kv_heads,
-                                head_dim, page_size, num_pages, scale, window, splits, waves, AttnExtras{sink, nullptr, 0}, s);
+                                head_dim, page_size, num_pages, scale, window, splits, waves, AttnExtras{sink, nullptr, 0, softcap}, s);
   return launch_decode<bf16_t>(q, q_stride, k_pool, v_pool, nullptr, 0, partial, tok_list,
                                tok_item, tok_pos, tables, table_width, count, heads, kv_heads,
-                               head_dim, page_size, num_pages, scale, window, splits, waves, AttnExtras{sink, nullptr, 0}, s);
+                               head_dim, page_size, num_pages, scale, window, splits, waves, AttnExtras{sink, nullptr, 0, softcap}, s);
 }
 
 extern "C" int ps_attention_decode(const void* q, int64_t q_stride, const void* k_pool,
@@ -236,7 +237,8 @@ extern "C" int ps_attention_decode(const void* q, int64_t q_stride, const void* 
                                    int table_width, int count, int heads, int kv_heads,
                                    int head_dim, int page_size, int num_pages, float scale,
                                    int window, int splits, int waves, const float* sink,
-                                   const float* gate, int64_t gate_ld, int dtype, void* stream) {
+                                   const float* gate, int64_t gate_ld, float softcap, int dtype,
+                                   void* stream) {
   if (check_decode_sizes("ps_attention_decode", count, heads, kv_heads, head_dim, page_size,
                          num_pages, table_width, window, splits, waves, dtype))
     return 1;
@@ -252,8 +254,8 @@ extern "C" int ps_attention_decode(const void* q, int64_t q_stride, const void* 
   if (dtype == PS_F32)
     return launch_decode<float>(q, q_stride, k_pool, v_pool, out, out_stride, partial, tok_list,
                                 tok_item, tok_pos, tables, table_width, count, heads, kv_heads,
-                                head_dim, page_size, num_pages, scale, window, splits, waves, AttnExtras{sink, gate, gate_ld}, s);
+                                head_dim, page_size, num_pages, scale, window, splits, waves, AttnExtras{sink, gate, gate_ld, softcap}, s);
   return launch_decode<bf16_t>(q, q_stride, k_pool, v_pool, out, out_stride, partial, tok_list,
                                tok_item, tok_pos, tables, table_width, count, heads, kv_heads,
-                               head_dim, page_size, num_pages, scale, window, splits, waves, AttnExtras{sink, gate, gate_ld}, s);
+                               head_dim, page_size, num_pages, scale, window, splits, waves, AttnExtras{sink, gate, gate_ld, softcap}, s);
 }

@@ -203,7 +203,10 @@ __device__ __forceinline__ void attention_decode_block(
         dot = lanes_sum<16>(dot);
         dot += __shfl_xor(dot, 16, 64);
       }
-      s[u] = valid[u] ? dot * scale_log2 : -INFINITY;
+      float score = dot * scale_log2;
+      // (the cap in the scores' units of log 2)
+      if (extra.softcap > 0.f) score = capped_score_as<T>(score, extra.softcap * 1.4426950408889634f);
+      s[u] = valid[u] ? score : -INFINITY;
       m_new = fmaxf(m_new, s[u]);
     }
     if (m_new != -INFINITY) {

@@ -76,7 +76,7 @@ extern "C" int ps_attention_mixed(const void* q, int64_t q_stride, const void* k
                                   const int* tables, int table_width, int heads, int kv_heads,
                                   int head_dim, int page_size, int num_pages, float scale,
                                   int window, const float* sink, const float* gate, int64_t gate_ld,
-                                  int dtype, void* stream) {
+                                  float softcap, int dtype, void* stream) {
   PS_REQUIRE(singles >= 0 && tiles >= 0 && heads > 0 && kv_heads > 0 && page_size > 0 &&
                  num_pages > 0 && table_width > 0,
              "ps_attention_mixed: bad sizes");
@@ -104,7 +104,7 @@ extern "C" int ps_attention_mixed(const void* q, int64_t q_stride, const void* k
     while ((1 << page_shift) < page_size) ++page_shift;
   }
   hipStream_t s = (hipStream_t)stream;
-  const AttnExtras extra = {sink, gate, gate_ld};
+  const AttnExtras extra = {sink, gate, gate_ld, softcap};
   const int decode_blocks = singles * heads;
   // as the decode kernel chooses: more blocks of its kind than compute units read their keys
   // without leaving lines in the caches

@@ -55,7 +55,8 @@ extern "C" int ps_attention_prefill(const void* q, int64_t q_stride, const void*
                                     int table_width, int heads, int kv_heads, int head_dim,
                                     int page_size, int num_pages, float scale, int window,
                                     int max_kv_len, int query_tile, const float* sink,
-                                    const float* gate, int64_t gate_ld, int dtype, void* stream) {
+                                    const float* gate, int64_t gate_ld, float softcap, int dtype,
+                                    void* stream) {
   PS_REQUIRE(tiles >= 0 && heads > 0 && kv_heads > 0 && page_size > 0 && num_pages > 0 &&
                  table_width > 0,
              "ps_attention_prefill: bad sizes");
@@ -86,7 +87,7 @@ extern "C" int ps_attention_prefill(const void* q, int64_t q_stride, const void*
     while ((1 << page_shift) < page_size) ++page_shift;
   }
   hipStream_t s = (hipStream_t)stream;
-  const AttnExtras extra = {sink, gate, gate_ld};
+  const AttnExtras extra = {sink, gate, gate_ld, softcap};
   dim3 grid(heads, tiles);
   // With few blocks, up to two per compute unit, which hold them all at once (128 registers and
   // 72 KB of LDS each), four waves along the keys shorten the longest block (2 x 1,024 tokens of

@@ -307,6 +307,14 @@ __device__ __forceinline__ void attention_prefill_block(
       const bool masked = kw + WAVE_KEYS - 1 > wave_first || kw + WAVE_KEYS > key_end ||
                           (window > 0 && kw < wave_last - window + 1) || !q_valid;
       // scores stay unscaled until the exponential: p = 2^(s c - m), with m kept in scaled units
+      if (extra.softcap > 0.f) {
+        // a cap on the scaled scores, in the unscaled scores' units
+        const float unit = extra.softcap / scale;
+#pragma unroll
+        for (int r = 0; r < KR; ++r)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) s[r][e] = capped_score_fast(s[r][e], unit);
+      }
       float tile_max = -INFINITY;
       if (__builtin_amdgcn_readfirstlane(__any(masked) ? 1 : 0)) {
 #pragma unroll

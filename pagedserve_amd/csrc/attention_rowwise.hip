@@ -60,6 +60,7 @@ __global__ __launch_bounds__(64) void attention_rowwise_kernel(
         float dot = 0.f;
         for (int i = 0; i < head_dim; ++i) dot = fmaf(q_row[i], to_float<T>(k_row[i]), dot);
         score = dot * scale;
+        if (extra.softcap > 0.f) score = capped_score(score, extra.softcap);
       }
     }
     const float chunk_max = wave_max(score);
@@ -105,7 +106,7 @@ extern "C" int ps_attention_rowwise(const void* q, int64_t q_stride, const void*
                                     int kv_heads,
                                     int head_dim, int page_size, int num_pages, float scale,
                                     int window, const float* sink, const float* gate,
-                                    int64_t gate_ld, int dtype, void* stream) {
+                                    int64_t gate_ld, float softcap, int dtype, void* stream) {
   PS_REQUIRE(tokens >= 0 && heads > 0 && kv_heads > 0 && page_size > 0 && num_pages > 0 &&
                  table_width > 0,
              "ps_attention_rowwise: bad sizes");
@@ -118,7 +119,7 @@ extern "C" int ps_attention_rowwise(const void* q, int64_t q_stride, const void*
   PS_REQUIRE(dtype == PS_F32 || dtype == PS_BF16, "ps_attention_rowwise: unknown dtype %d", dtype);
   if (tokens == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
-  const AttnExtras extra = {sink, gate, gate_ld};
+  const AttnExtras extra = {sink, gate, gate_ld, softcap};
   dim3 grid(tokens, heads);
   if (dtype == PS_F32)
     hipLaunchKernelGGL(attention_rowwise_kernel<float>, grid, dim3(64), 0, s, (const float*)q,

@@ -146,7 +146,9 @@ __global__ __launch_bounds__(256) void attention_tiled_f32_kernel(
       for (int j = 0; j < 4; ++j) {
         const int key = k0 + tx + 16 * j;
         const bool visible = key_ok[j] && key <= q_pos[i] && (window <= 0 || q_pos[i] - key < window);
-        s[i][j] = visible ? s[i][j] * scale : -INFINITY;
+        float score = s[i][j] * scale;
+        if (extra.softcap > 0.f) score = capped_score(score, extra.softcap);
+        s[i][j] = visible ? score : -INFINITY;
         tile_max = fmaxf(tile_max, s[i][j]);
       }
       // the 16 threads of a row are 16 neighbouring lanes of one wave
@@ -236,7 +238,7 @@ extern "C" int ps_attention_tiled_f32(const void* q, int64_t q_stride, const voi
                                       int table_width, int heads, int kv_heads, int head_dim,
                                       int page_size, int num_pages, float scale, int window,
                                       const float* sink, const float* gate, int64_t gate_ld,
-                                      void* stream) {
+                                      float softcap, void* stream) {
   PS_REQUIRE(tiles >= 0 && heads > 0 && kv_heads > 0 && page_size > 0 && num_pages > 0 &&
                  table_width > 0,
              "ps_attention_tiled_f32: bad sizes");
@@ -254,7 +256,7 @@ extern "C" int ps_attention_tiled_f32(const void* q, int64_t q_stride, const voi
   PS_REQUIRE(blocks < ((int64_t)1 << 31), "ps_attention_tiled_f32: too many blocks");
   if (blocks == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
-  const AttnExtras extra = {sink, gate, gate_ld};
+  const AttnExtras extra = {sink, gate, gate_ld, softcap};
 #define PS_LAUNCH_AF(DV)                                                                          \
   hipLaunchKernelGGL(attention_tiled_f32_kernel<DV>, dim3((unsigned)blocks), dim3(256), 0, s,     \
                      (const float*)q, q_stride, (const float*)k_pool, (const float*)v_pool,       \

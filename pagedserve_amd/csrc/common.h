@@ -211,13 +211,32 @@ __device__ inline float apply_activation(float v) {
 }
 
 // What an attention kernel may be given beside its operands: a sink (one float per head whose
-// exponential joins the softmax's denominator; null: none) and a gate (the output of token t
-// and head h is multiplied by sigmoid(gate[t * gate_ld + h]); null: none).
+// exponential joins the softmax's denominator; null: none), a gate (the output of token t
+// and head h is multiplied by sigmoid(gate[t * gate_ld + h]); null: none) and a cap on the
+// scaled scores (s <- cap * tanh(s / cap) before the softmax; 0: none).
 struct AttnExtras {
   const float* sink;
   const float* gate;
   long long gate_ld;
+  float softcap;
 };
+
+// c * tanh(s / c), with the score and the cap in the same units (a kernel that keeps scores
+// unscaled, or in units of log 2, hands over the cap divided or multiplied accordingly).
+__device__ inline float capped_score(float s, float cap) { return cap * tanhf(s / cap); }
+
+// The same from the hardware's exponential and reciprocal, tanh(x) = 1 - 2 / (1 + e^(2x)): for
+// kernels whose scores feed bfloat16 products (absolute error of some 1e-7 of the cap).
+__device__ inline float capped_score_fast(float s, float cap) {
+  const float e = __builtin_amdgcn_exp2f(s * __builtin_amdgcn_rcpf(cap) * 2.885390081777927f);
+  return cap * (1.f - 2.f * __builtin_amdgcn_rcpf(1.f + e));
+}
+template <typename T>
+__device__ inline float capped_score_as(float s, float cap);
+template <>
+__device__ inline float capped_score_as<float>(float s, float cap) { return capped_score(s, cap); }
+template <>
+__device__ inline float capped_score_as<bf16_t>(float s, float cap) { return capped_score_fast(s, cap); }
 
 __device__ inline float gate_factor(const AttnExtras& extra, long long token, int head) {
   if (extra.gate == nullptr) return 1.f;

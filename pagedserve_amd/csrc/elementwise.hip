@@ -51,14 +51,17 @@ int ps_compute_units() {
 
 // ---------------------------------------------------------------- embedding
 // h0[t] = scale * wte[id[t]] + wpe[pos[t]]  (reference: src/model/paged_decoder.py:306-314,
-// where the scale is 1).
+// where the scale is 1); with norm_gamma, the row is then RMS-normed in float in the same
+// launch: h0 <- h0 / sqrt(mean(h0^2) + eps) * norm_gamma.
 // The id of token t is ids[t], or carried[src[t]] where src[t] >= 0: a token that an earlier
 // step chose on the device and that the host has not seen yet.
 template <typename T>
 __global__ void embed_kernel(const T* __restrict__ table, const T* __restrict__ pos_table,
                              const int* __restrict__ ids, const int* __restrict__ src,
                              const int* __restrict__ carried, const int* __restrict__ positions,
-                             float* __restrict__ out, int width, int vocab, float scale) {
+                             float* __restrict__ out, int width, int vocab, float scale,
+                             const float* __restrict__ norm_gamma, float norm_eps) {
+  __shared__ float scratch[16];
   const int t = blockIdx.x;
   int id = ids[t];
   if (src != nullptr) {
@@ -75,28 +78,35 @@ __global__ void embed_kernel(const T* __restrict__ table, const T* __restrict__ 
   } else {
     for (int i = threadIdx.x; i < width; i += blockDim.x) dst[i] = to_float<T>(row[i]) * scale;
   }
+  if (norm_gamma == nullptr) return;
+  // (each thread reads back what it wrote itself)
+  float sum = 0.f;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) sum = fmaf(dst[i], dst[i], sum);
+  const float inv = 1.0f / sqrtf(block_sum(sum, scratch) / (float)width + norm_eps);
+  for (int i = threadIdx.x; i < width; i += blockDim.x) dst[i] = dst[i] * inv * norm_gamma[i];
 }
 
 extern "C" int ps_embed(const void* table, const void* pos_table, const int* ids, const int* src,
                         const int* carried, const int* positions, float* out, int tokens,
-                        int width, int vocab, int max_positions, float scale, int dtype,
-                        void* stream) {
+                        int width, int vocab, int max_positions, float scale,
+                        const float* norm_gamma, float norm_eps, int dtype, void* stream) {
   PS_REQUIRE(tokens >= 0 && width > 0 && vocab > 0, "ps_embed: bad sizes (tokens %d, width %d)",
              tokens, width);
   PS_REQUIRE(dtype == PS_F32 || dtype == PS_BF16, "ps_embed: unknown dtype %d", dtype);
   PS_REQUIRE(pos_table == nullptr || max_positions > 0, "ps_embed: position table without rows");
   PS_REQUIRE(src == nullptr || carried != nullptr, "ps_embed: carried tokens are missing");
+  PS_REQUIRE(norm_gamma == nullptr || norm_eps > 0.f, "ps_embed: a norm needs a positive eps");
   if (tokens == 0) return 0;
   const int threads = width >= 256 ? 256 : 64;
   hipStream_t s = (hipStream_t)stream;
   if (dtype == PS_F32)
     hipLaunchKernelGGL(embed_kernel<float>, dim3(tokens), dim3(threads), 0, s, (const float*)table,
                        (const float*)pos_table, ids, src, carried, positions, out, width, vocab,
-                       scale);
+                       scale, norm_gamma, norm_eps);
   else
     hipLaunchKernelGGL(embed_kernel<bf16_t>, dim3(tokens), dim3(threads), 0, s,
                        (const bf16_t*)table, (const bf16_t*)pos_table, ids, src, carried,
-                       positions, out, width, vocab, scale);
+                       positions, out, width, vocab, scale, norm_gamma, norm_eps);
   PS_CHECK_LAUNCH("ps_embed");
   return 0;
 }

@@ -21,10 +21,12 @@ const char* ps_last_error(void);
 int ps_device_info(int* compute_units, int* lds_bytes, char* arch, int arch_len);
 
 // out[t, :] = scale * table[id(t), :] + (pos_table ? pos_table[positions[t], :] : 0), in float,
-// where id(t) = ids[t], or carried[src[t]] if src is given and src[t] >= 0.
+// where id(t) = ids[t], or carried[src[t]] if src is given and src[t] >= 0.  norm_gamma (null:
+// none): the row is then RMS-normed, out / sqrt(mean(out^2) + norm_eps) * norm_gamma.
 int ps_embed(const void* table, const void* pos_table, const int* ids, const int* src,
              const int* carried, const int* positions, float* out, int tokens, int width,
-             int vocab, int max_positions, float scale, int dtype, void* stream);
+             int vocab, int max_positions, float scale, const float* norm_gamma, float norm_eps,
+             int dtype, void* stream);
 
 // out[r, :] = norm(x[rows ? rows[r] : r, :]) * gamma (+ beta).  rms != 0: no mean, no beta.
 int ps_norm(const float* x, const int* rows, const float* gamma, const float* beta, void* out,
@@ -118,13 +120,14 @@ int ps_kv_write(const void* k, const void* v, int64_t stride, void* k_pool, void
 // (a score without key or value, not scaled); gate: null, or a float per token and head, rows
 // gate_ld apart: the output of token t and head h is multiplied by sigmoid(gate[t * gate_ld + h]);
 // the same in the attention kernels below (ps_attention_decode_partial leaves the gate to
-// whoever merges its records).
+// whoever merges its records).  softcap: 0, or c > 0: a scaled score s enters the softmax as
+// c * tanh(s / c).
 int ps_attention_rowwise(const void* q, int64_t q_stride, const void* k_pool, const void* v_pool,
                          void* out, int64_t out_stride, const int* tok_list, const int* tok_item,
                          const int* tok_pos, const int* tables, int table_width, int tokens,
                          int heads, int kv_heads, int head_dim, int page_size, int num_pages,
                          float scale, int window, const float* sink, const float* gate,
-                         int64_t gate_ld, int dtype, void* stream);
+                         int64_t gate_ld, float softcap, int dtype, void* stream);
 
 // The same result in true 32-bit for the items of several tokens (prompt portions), a block
 // of four waves per (tile of ps_attention_tiled_f32_tile() queries, head): float pools, float
@@ -138,7 +141,7 @@ int ps_attention_tiled_f32(const void* q, int64_t q_stride, const void* k_pool, 
                            int tiles, const int* cu_tokens, const int* kv_lens, const int* tables,
                            int table_width, int heads, int kv_heads, int head_dim, int page_size,
                            int num_pages, float scale, int window, const float* sink, const float* gate,
-                           int64_t gate_ld, void* stream);
+                           int64_t gate_ld, float softcap, void* stream);
 
 // The same result for single queries, with each token's keys cut into `splits` ranges that
 // run as separate blocks of `waves` (4 or 16) waves; `partial` is scratch of
@@ -152,7 +155,7 @@ int ps_attention_decode(const void* q, int64_t q_stride, const void* k_pool, con
                         const int* tables, int table_width, int count, int heads, int kv_heads,
                         int head_dim, int page_size, int num_pages, float scale, int window,
                         int splits, int waves, const float* sink, const float* gate, int64_t gate_ld,
-                        int dtype, void* stream);
+                        float softcap, int dtype, void* stream);
 
 // Only the records of ps_attention_decode: (unnormalised sum of values [head_dim], maximum in
 // units of log 2, sum) per (token, head, range) at partial[((n * heads + head) * splits + s) *
@@ -163,7 +166,7 @@ int ps_attention_decode_partial(const void* q, int64_t q_stride, const void* k_p
                                 const int* tables, int table_width, int count, int heads,
                                 int kv_heads, int head_dim, int page_size, int num_pages,
                                 float scale, int window, int splits, int waves, const float* sink,
-                                int dtype, void* stream);
+                                float softcap, int dtype, void* stream);
 
 // The merge of those records inside the output projection, for up to 16 tokens and head sizes
 // that are multiples of 64 (bfloat16 weights in their packed copy, n output columns,
@@ -209,8 +212,8 @@ int ps_attention_prefill(const void* q, int64_t q_stride, const void* k_pool, co
                          int tiles, const int* cu_tokens, const int* kv_lens, const int* tables,
                          int table_width, int heads, int kv_heads, int head_dim, int page_size,
                          int num_pages, float scale, int window, int max_kv_len, int query_tile,
-                         const float* sink, const float* gate, int64_t gate_ld, int dtype,
-                         void* stream);
+                         const float* sink, const float* gate, int64_t gate_ld, float softcap,
+                         int dtype, void* stream);
 
 // Both of the above in one launch, for a step that has items of one token (tok_list lists the
 // `singles` tokens; tok_item and tok_pos are indexed by token as in ps_attention_decode, which
@@ -225,7 +228,7 @@ int ps_attention_mixed(const void* q, int64_t q_stride, const void* k_pool, cons
                        const int* tile_q0, int tiles, const int* cu_tokens, const int* kv_lens,
                        const int* tables, int table_width, int heads, int kv_heads, int head_dim,
                        int page_size, int num_pages, float scale, int window, const float* sink,
-                       const float* gate, int64_t gate_ld, int dtype, void* stream);
+                       const float* gate, int64_t gate_ld, float softcap, int dtype, void* stream);
 
 // The constants of that kernel that a caller builds its index arrays by: queries per tile (of
 // the two sizes), and the widest block table (entries per item) that it takes.
@@ -276,6 +279,29 @@ int ps_attention_prepare(const float* proj, int64_t ld, int q_col, int k_col, in
                          int table_width, int tokens, int heads, int kv_heads, int key_dim,
                          int value_dim, int cache_dim, int page_size, int num_pages, int dtype,
                          void* stream);
+// The same step for layers that treat every head on its own: the first rot_dims dimensions of
+// each query and key head rotated (halves != 0: dimension i with i + rot_dims / 2, else 2i with
+// 2i + 1; cosine and sine times magnitude), then, with head_norm, every head divided by its root
+// mean square over key_dim (no weight); values: the columns at v_col as projected (v_col may be
+// k_col: values that are the keys before rotation and norm).  cache_dim up to 256.
+int ps_attention_prepare_heads(const float* proj, int64_t ld, int q_col, int k_col, int v_col,
+                               void* q_out, int64_t q_stride, void* k_pool, void* v_pool,
+                               const float* freqs, int rot_dims, int halves, float magnitude,
+                               int head_norm, float eps, const int* tok_item, const int* tok_pos,
+                               const int* tables, int table_width, int tokens, int heads,
+                               int kv_heads, int key_dim, int value_dim, int cache_dim,
+                               int page_size, int num_pages, int dtype, void* stream);
+// Latent attention: proj holds per head [dim | rot_dims] query dimensions from q_col on and, from
+// kv_col on, a latent of `rank` numbers and one rotated key part of rot_dims.  The token's one
+// cached row (k_pool: [pages, 1, page, cache_dim]) becomes [rms_norm(latent) * gamma | rotated key
+// part | zeros]; of every head's query row (cache_dim wide) the places rank .. rank + rot_dims - 1
+// get the rotated query part and the places behind zeros (the first `rank` are the caller's).
+int ps_latent_prepare(const float* proj, int64_t ld, int q_col, int kv_col, void* q_out,
+                      int64_t q_stride, void* k_pool, const float* gamma, float eps,
+                      const float* freqs, int rot_dims, int halves, float magnitude,
+                      const int* tok_item, const int* tok_pos, const int* tables, int table_width,
+                      int tokens, int heads, int dim, int rank, int cache_dim, int page_size,
+                      int num_pages, int dtype, void* stream);
 // ctx[t, h, :] *= sigmoid(gate[t * gate_ld + h]).
 int ps_head_gate(void* ctx, int64_t stride, const float* gate, int64_t gate_ld, int tokens,
                  int heads, int head_dim, int dtype, void* stream);
@@ -320,12 +346,12 @@ int ps_softcap(float* logits, int64_t ld, int rows, int vocab, float cap, void* 
 // ---- selective state-space mixer -------------------------------------------------------------
 // state: [slots, channels, states + taps - 1] float per request: the recurrence's numbers of a
 // channel and behind them its last taps - 1 raw inputs, oldest first.
-// x[t, c] = silu(bias[c] + sum_j w[c, j] u[t - taps + 1 + j, c]) with u = proj[:, u_col + c]; inputs
-// from before the step come from the slot.
+// x[t, c] = act(bias[c] + sum_j w[c, j] u[t - taps + 1 + j, c]) with u = proj[:, u_col + c]; inputs
+// from before the step come from the slot.  activation: 1 silu, 0 none.  dtype: that of x.
 int ps_conv_silu(const float* proj, int64_t ld, int u_col, const float* w, const float* bias,
                  const float* state, int states, void* x, const int* tok_item,
                  const int* cu_tokens, const int* slots, int tokens, int channels, int taps,
-                 int dtype, void* stream);
+                 int activation, int dtype, void* stream);
 // dt[t, c] = softplus(bias[c] + sum_r low[t * ld + r] w[c, r]) in float.
 int ps_step_size(const float* low, int64_t ld, int rank, const void* w, const float* bias, float* dt,
                  int tokens, int channels, int dtype, void* stream);
@@ -346,11 +372,12 @@ int ps_selective_scan(const void* x, const float* dt, const float* bc, int64_t b
                       const float* step_bias, int low_col, int rank, int dtype, void* stream);
 
 // ---- a stream whose sublayers add into a scratch row ------------------------------------------
-// h += factor * y + bias (y, bias: null for none); zero[...] = 0 (may be y); if gamma:
+// h += factor * column_scale * y + bias (y, bias: null for none; column_scale: a float per
+// column, null for ones); zero[...] = 0 (may be y); if gamma:
 // normed = h / sqrt(mean(h^2) + eps) * gamma.
-int ps_stream_step(float* h, const float* y, float factor, const float* bias, const float* gamma,
-                   float eps, void* normed, float* zero, int tokens, int width, int out_dtype,
-                   void* stream);
+int ps_stream_step(float* h, const float* y, float factor, const float* column_scale,
+                   const float* bias, const float* gamma, float eps, void* normed, float* zero,
+                   int tokens, int width, int out_dtype, void* stream);
 // out[t, c] = silu(gu[t * ld + c]) * gu[t * ld + inner + c].
 int ps_silu_gate(const float* gu, int64_t ld, void* out, int64_t out_ld, int tokens, int inner,
                  int dtype, void* stream);
@@ -359,6 +386,28 @@ int ps_silu_columns(float* p, int64_t ld, int first, int count, int tokens, void
 // y += share * (rms_norm(a) * wa + rms_norm(b) * wb) over rows of width floats; a and b are cleared.
 int ps_pair_norm_mix(float* a, float* b, const float* wa, const float* wb, float eps, float share,
                      float* y, int tokens, int width, void* stream);
+
+// ---- block-diagonal products -------------------------------------------------------------------
+// out[t, b * out_step + j] = (sum_i x[t, b * x_step + i] w[b, j, i] + bias[b * n + j])
+//                            * (gate ? sigmoid(gate[t * gate_ld + b * n + j]) : 1)
+// for `blocks` matrices w[b] of [n, k]; x and out float or bfloat16 rows (x_ld, out_ld apart),
+// w bfloat16, or everything float.
+int ps_block_linear(const void* x, int x_dtype, int64_t x_ld, int x_step, const void* w, int w_dtype,
+                    const float* bias, void* out, int out_dtype, int64_t out_ld, int out_step,
+                    const float* gate, int64_t gate_ld, int blocks, int n, int k, int tokens,
+                    void* stream);
+
+// ---- gated linear recurrence with one state per channel ---------------------------------------
+// state: [slots, channels, taps] float per request: S and behind it the last taps - 1 raw inputs
+// of the short convolution (proj[:, x_col + c], oldest first).  Per item, token after token:
+// a = exp(-decay_scale * sigmoid(gr[t, c]) * softplus(lam[c])),
+// S = a S + sqrt(1 - a^2) sigmoid(gi[t, c]) u[t, c],
+// out[t, c] = S * gelu_tanh(proj[t, y_col + c]); a row of gates (2 * channels floats) holds, for
+// every run of `block` channels, their gr and then their gi.
+int ps_lru_scan(const float* proj, int64_t ld, int y_col, int x_col, const float* u,
+                const float* gates, int block, const float* lam, float decay_scale, float* state, void* out,
+                const int* cu_tokens, const int* slots, int items, int tokens, int channels,
+                int taps, int dtype, void* stream);
 
 // ---- mixture of experts ------------------------------------------------------------------------
 // ids / weights [tokens, top]: the experts that each row of x chooses and s * scale of each

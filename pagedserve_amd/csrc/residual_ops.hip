@@ -6,19 +6,20 @@
 #include "pagedserve_hip.h"
 
 // One pass over the stream's rows, every piece optional:
-//   h <- h + factor * y + bias;   zero <- 0 (may be y);   normed <- h / sqrt(mean(h^2) + eps) * gamma
-// A block per token.
+//   h <- h + factor * column_scale * y + bias;   zero <- 0 (may be y);
+//   normed <- h / sqrt(mean(h^2) + eps) * gamma
+// (column_scale: a float per column, null for ones).  A block per token.
 template <typename T>
 __global__ __launch_bounds__(256) void stream_step_kernel(
-    float* __restrict__ h, const float* y, float factor, const float* __restrict__ bias,
-    const float* __restrict__ gamma, float eps, T* __restrict__ normed, float* zero, int width) {
+    float* __restrict__ h, const float* y, float factor, const float* __restrict__ column_scale,
+    const float* __restrict__ bias, const float* __restrict__ gamma, float eps, T* __restrict__ normed, float* zero, int width) {
   __shared__ float scratch[16];
   const int64_t t = blockIdx.x;
   float* row = h + t * width;
   float sum = 0.f;
   for (int d = threadIdx.x; d < width; d += blockDim.x) {
     float v = row[d];
-    if (y != nullptr) v = fmaf(factor, y[t * width + d], v);
+    if (y != nullptr) v = fmaf(column_scale ? factor * column_scale[d] : factor, y[t * width + d], v);
     if (bias != nullptr) v += bias[d];
     if (y != nullptr || bias != nullptr) row[d] = v;
     if (zero != nullptr) zero[t * width + d] = 0.f;
@@ -78,9 +79,9 @@ __global__ __launch_bounds__(256) void pair_norm_mix_kernel(
   }
 }
 
-extern "C" int ps_stream_step(float* h, const float* y, float factor, const float* bias,
-                              const float* gamma, float eps, void* normed, float* zero, int tokens,
-                              int width, int out_dtype, void* stream) {
+extern "C" int ps_stream_step(float* h, const float* y, float factor, const float* column_scale,
+                              const float* bias, const float* gamma, float eps, void* normed,
+                              float* zero, int tokens, int width, int out_dtype, void* stream) {
   PS_REQUIRE(tokens >= 0 && width > 0, "ps_stream_step: bad sizes");
   PS_REQUIRE(gamma == nullptr || (normed != nullptr && eps > 0.f),
              "ps_stream_step: a norm needs an output and a positive eps");
@@ -88,11 +89,11 @@ extern "C" int ps_stream_step(float* h, const float* y, float factor, const floa
   if (tokens == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
   if (out_dtype == PS_F32)
-    hipLaunchKernelGGL(stream_step_kernel<float>, dim3(tokens), dim3(256), 0, s, h, y, factor, bias,
-                       gamma, eps, (float*)normed, zero, width);
+    hipLaunchKernelGGL(stream_step_kernel<float>, dim3(tokens), dim3(256), 0, s, h, y, factor,
+                       column_scale, bias, gamma, eps, (float*)normed, zero, width);
   else
-    hipLaunchKernelGGL(stream_step_kernel<bf16_t>, dim3(tokens), dim3(256), 0, s, h, y, factor, bias,
-                       gamma, eps, (bf16_t*)normed, zero, width);
+    hipLaunchKernelGGL(stream_step_kernel<bf16_t>, dim3(tokens), dim3(256), 0, s, h, y, factor,
+                       column_scale, bias, gamma, eps, (bf16_t*)normed, zero, width);
   PS_CHECK_LAUNCH("ps_stream_step");
   return 0;
 }

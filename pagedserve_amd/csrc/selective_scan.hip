@@ -44,7 +44,7 @@ __global__ __launch_bounds__(256) void conv_silu_kernel(
     const float* __restrict__ proj, int64_t ld, int u_col, const float* __restrict__ w,
     const float* __restrict__ bias, const float* __restrict__ state, int row, int tail,
     T* __restrict__ x, const int* __restrict__ tok_item, const int* __restrict__ cu_tokens,
-    const int* __restrict__ slots, int channels, int taps) {
+    const int* __restrict__ slots, int channels, int taps, int activation) {
   const int t = blockIdx.x;
   const int c = blockIdx.y * 256 + threadIdx.x;
   if (c >= channels) return;
@@ -59,7 +59,7 @@ __global__ __launch_bounds__(256) void conv_silu_kernel(
                                : kept[taps - 1 + local];
     sum = fmaf(w[(int64_t)c * taps + j], u, sum);
   }
-  x[(int64_t)t * channels + c] = from_float<T>(silu_f(sum));
+  x[(int64_t)t * channels + c] = from_float<T>(activation ? silu_f(sum) : sum);
 }
 
 // dt[t, c] = softplus(bias[c] + sum_r low[t, r] w[c, r]).  A thread per channel and SS_STEP_TOKENS
@@ -367,7 +367,7 @@ __global__ __launch_bounds__(256) void selective_join_kernel(ScanArgs p, float* 
 extern "C" int ps_conv_silu(const float* proj, int64_t ld, int u_col, const float* w,
                             const float* bias, const float* state, int states, void* x,
                             const int* tok_item, const int* cu_tokens, const int* slots, int tokens,
-                            int channels, int taps, int dtype, void* stream) {
+                            int channels, int taps, int activation, int dtype, void* stream) {
   PS_REQUIRE(tokens >= 0 && channels > 0 && taps >= 1 && taps <= 64 && states >= 0,
              "ps_conv_silu: bad sizes");
   PS_REQUIRE(dtype == PS_F32 || dtype == PS_BF16, "ps_conv_silu: unknown dtype %d", dtype);
@@ -377,10 +377,10 @@ extern "C" int ps_conv_silu(const float* proj, int64_t ld, int u_col, const floa
   const int row = states + taps - 1;
   if (dtype == PS_F32)
     hipLaunchKernelGGL(conv_silu_kernel<float>, grid, dim3(256), 0, s, proj, ld, u_col, w, bias, state,
-                       row, states, (float*)x, tok_item, cu_tokens, slots, channels, taps);
+                       row, states, (float*)x, tok_item, cu_tokens, slots, channels, taps, activation);
   else
     hipLaunchKernelGGL(conv_silu_kernel<bf16_t>, grid, dim3(256), 0, s, proj, ld, u_col, w, bias, state,
-                       row, states, (bf16_t*)x, tok_item, cu_tokens, slots, channels, taps);
+                       row, states, (bf16_t*)x, tok_item, cu_tokens, slots, channels, taps, activation);
   PS_CHECK_LAUNCH("ps_conv_silu");
   return 0;
 }

@@ -51,6 +51,14 @@ class DecoderModel:
             self.blocks.append(arrangement(width=spec.width, dtype=dtype, parts=parts,
                                            **dict(block_spec.params)))
         self.final_norm = build_part(NORMS, "norm", spec.final_norm, **common)
+        self.embedding_norm = None
+        if spec.embedding_norm is not None:
+            # normed in the embedding's own launch: an RMS norm without a shift, of one stream
+            self.embedding_norm = build_part(NORMS, "norm", spec.embedding_norm, **common)
+            if (not hasattr(self.embedding_norm, "gamma_eps") or spec.streams
+                    or not getattr(self.embedding, "takes_norm", False)):
+                raise ValueError("the embedding's norm must be an RMS norm without a shift, on a single "
+                                 "stream, with an embedding that norms in its own launch")
         # Queries of a prompt portion are handed to the mixers in tiles; each mixer says which
         # size (or sizes) its kernel takes, and the step lists the tiles once per size that is
         # asked for.
@@ -85,6 +93,8 @@ class DecoderModel:
     def _named_parts(self):
         """(prefix of the parameter paths, part) of every part that may own parameters."""
         yield "embedding.", self.embedding
+        if self.embedding_norm is not None:
+            yield "embedding_norm.", self.embedding_norm
         yield "position.", self.position
         if self.spec.pass_rows:
             yield "", self
@@ -135,14 +145,14 @@ class DecoderModel:
                 flat.append((entry, spec))
         for entry, spec in flat:
             if isinstance(spec, PagedKVSpec):
-                by_geometry.setdefault((spec.kv_heads, spec.head_dim, spec.window, spec.value_dim),
-                                       []).append(entry)
+                by_geometry.setdefault((spec.kv_heads, spec.head_dim, spec.window, spec.value_dim,
+                                        spec.values_in_keys), []).append(entry)
             elif isinstance(spec, SlotStateSpec):
                 states.append(StateSpec(entry, tuple(spec.shape), spec.dtype))
             elif spec is not None:
                 raise TypeError(f"unknown cache spec {spec!r}")
-        groups = [CacheGroupSpec(tuple(entries), kv_heads, head_dim, window, value_dim)
-                  for (kv_heads, head_dim, window, value_dim), entries in by_geometry.items()]
+        groups = [CacheGroupSpec(tuple(entries), kv_heads, head_dim, window, value_dim, shared)
+                  for (kv_heads, head_dim, window, value_dim, shared), entries in by_geometry.items()]
         return groups, states
 
     def cache_views(self, cache) -> List[CacheView]:
@@ -174,6 +184,8 @@ class DecoderModel:
         """Whether a step of this model may be recorded and replayed as a graph: every part
         says so of itself."""
         parts = [self.embedding, self.position, self.final_norm, self.head] + list(self.blocks)
+        if self.embedding_norm is not None:
+            parts.append(self.embedding_norm)
         return all(getattr(part, "graph_safe", False) for part in parts)
 
     def forward(self, ctx, views, logit_rows, logits_out, choose=None):
@@ -192,7 +204,11 @@ class DecoderModel:
             kernels.streams_expand(embedded, h, tokens, width, streams)
         else:
             h = ctx.workspace.first_rows("residual", width, torch.float32, tokens)
-            self.embedding.forward(ctx, self.position.embedding_table(), h)
+            if self.embedding_norm is not None:
+                self.embedding.forward(ctx, self.position.embedding_table(), h,
+                                       norm=self.embedding_norm.gamma_eps())
+            else:
+                self.embedding.forward(ctx, self.position.embedding_table(), h)
         schedule = self.spec.schedule
         for index, (call, view) in enumerate(zip(schedule, views)):
             block = self.blocks[call.block]

@@ -22,7 +22,7 @@ _DTYPE_CODE = {torch.float32: F32, torch.bfloat16: BF16}
 
 _SIGNATURES = {
     "ps_embed": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
-                 c_int, c_int, c_int, c_float, c_int, c_void_p],
+                 c_int, c_int, c_int, c_float, c_void_p, c_float, c_int, c_void_p],
     "ps_norm": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_float, c_int,
                 c_int, c_void_p],
     "ps_gemm_nt": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
@@ -31,7 +31,8 @@ _SIGNATURES = {
                     c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "ps_attention_rowwise": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p,
                              c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
-                             c_int, c_float, c_int, c_void_p, c_void_p, c_int64, c_int, c_void_p],
+                             c_int, c_float, c_int, c_void_p, c_void_p, c_int64, c_float, c_int,
+                             c_void_p],
     "ps_hyper_step": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_void_p,
                       c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     "ps_streams_expand": [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
@@ -52,15 +53,26 @@ _SIGNATURES = {
     "ps_row_norm_gate": [c_void_p, c_void_p, c_float, c_void_p, c_int64, c_void_p, c_int64, c_int,
                          c_int, c_int, c_void_p],
     "ps_conv_silu": [c_void_p, c_int64, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
-                     c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+                     c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "ps_attention_prepare_heads": [c_void_p, c_int64, c_int, c_int, c_int, c_void_p, c_int64, c_void_p,
+                                   c_void_p, c_void_p, c_int, c_int, c_float, c_int, c_float, c_void_p,
+                                   c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+                                   c_int, c_int, c_int, c_void_p],
+    "ps_latent_prepare": [c_void_p, c_int64, c_int, c_int, c_void_p, c_int64, c_void_p, c_void_p,
+                          c_float, c_void_p, c_int, c_int, c_float, c_void_p, c_void_p, c_void_p, c_int,
+                          c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "ps_block_linear": [c_void_p, c_int, c_int64, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int,
+                        c_int64, c_int, c_void_p, c_int64, c_int, c_int, c_int, c_int, c_void_p],
+    "ps_lru_scan": [c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_float, c_void_p,
+                    c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "ps_step_size": [c_void_p, c_int64, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                      c_void_p],
     "ps_selective_scan": [c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p, c_int64,
                           c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                           c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                           c_int, c_int, c_int, c_void_p],
-    "ps_stream_step": [c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_float, c_void_p, c_void_p,
-                       c_int, c_int, c_int, c_void_p],
+    "ps_stream_step": [c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_float, c_void_p,
+                       c_void_p, c_int, c_int, c_int, c_void_p],
     "ps_silu_columns": [c_void_p, c_int64, c_int, c_int, c_int, c_void_p],
     "ps_silu_gate": [c_void_p, c_int64, c_void_p, c_int64, c_int, c_int, c_int, c_void_p],
     "ps_pair_norm_mix": [c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_float, c_void_p, c_int,
@@ -78,23 +90,25 @@ _SIGNATURES = {
     "ps_attention_decode": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p,
                             c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                             c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_void_p, c_void_p,
-                            c_int64, c_int, c_void_p],
+                            c_int64, c_float, c_int, c_void_p],
     "ps_attention_decode_partial": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p,
                                     c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
-                                    c_int, c_int, c_float, c_int, c_int, c_int, c_void_p, c_int, c_void_p],
+                                    c_int, c_int, c_float, c_int, c_int, c_int, c_void_p, c_float, c_int,
+                                    c_void_p],
     "ps_attention_merge_linear": [c_void_p, c_int64, c_void_p, c_int, c_int, c_int, c_int, c_void_p,
                                   c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p],
     "ps_attention_tiled_f32": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p,
                                c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
-                               c_int, c_int, c_int, c_float, c_int, c_void_p, c_void_p, c_int64, c_void_p],
+                               c_int, c_int, c_int, c_float, c_int, c_void_p, c_void_p, c_int64, c_float,
+                               c_void_p],
     "ps_attention_prefill": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p,
                              c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                              c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_void_p, c_void_p, c_int64,
-                             c_int, c_void_p],
+                             c_float, c_int, c_void_p],
     "ps_attention_mixed": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int,
                            c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
                            c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p, c_void_p,
-                           c_int64, c_int, c_void_p],
+                           c_int64, c_float, c_int, c_void_p],
     "ps_sample": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
 }
 
@@ -183,10 +197,11 @@ def _ptr(tensor):
     return 0 if tensor is None else tensor.data_ptr()
 
 
-def embed(table, pos_table, ids, positions, out, token_src=None, carried=None, scale=1.0):
+def embed(table, pos_table, ids, positions, out, token_src=None, carried=None, scale=1.0, norm=None):
     """out[t] = scale * table[id(t)] + pos_table[positions[t]] as float (pos_table may be None).
     id(t) is ``ids[t]``, or ``carried[token_src[t]]`` where ``token_src[t] >= 0``: a token
-    that an earlier step chose on the device."""
+    that an earlier step chose on the device.  ``norm = (gamma, eps)``: every row is then
+    RMS-normed in the same launch, ``out / sqrt(mean(out^2) + eps) * gamma``."""
     _check(table, "table", ndim=2)
     _check(ids, "ids", torch.int32, 1)
     _check(out, "out", torch.float32, 2)
@@ -210,10 +225,15 @@ def embed(table, pos_table, ids, positions, out, token_src=None, carried=None, s
         _check(carried, "carried", torch.int32, 1)
         if token_src.numel() != tokens or not token_src.is_contiguous() or not carried.is_contiguous():
             raise KernelError("embed: one source index per token is needed")
+    gamma, eps = None, 1.0
+    if norm is not None:
+        gamma, eps = norm
+        _float_vector(gamma, "norm gamma", width)
     _call("ps_embed", table.data_ptr(), _ptr(pos_table), ids.data_ptr(), _ptr(token_src),
           _ptr(carried if token_src is not None else None),
           _ptr(positions if pos_table is not None else None), out.data_ptr(), tokens, width,
-          table.shape[0], max_positions, float(scale), dtype_code(table.dtype), _stream())
+          table.shape[0], max_positions, float(scale), _ptr(gamma), float(eps),
+          dtype_code(table.dtype), _stream())
     return out
 
 
@@ -696,8 +716,16 @@ def _check_gate(gate, tokens, heads):
     return gate.data_ptr(), _rows(gate, "gate")
 
 
+def _check_cap(softcap):
+    """A cap ``c > 0`` on the scaled scores (``c tanh(s / c)`` enters the softmax), or 0 for none."""
+    softcap = float(softcap or 0.0)
+    if not softcap >= 0.0 or softcap == float("inf"):
+        raise KernelError(f"attention: a score cap must be positive and finite (0: none), got {softcap}")
+    return softcap
+
+
 def attention_rowwise(q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, scale, window=0,
-                      tok_list=None, sink=None, gate=None):
+                      tok_list=None, sink=None, gate=None, softcap=0.0):
     """out[t, h] = softmax(q[t, h] . K * scale) V over the cached keys of t's request, for the
     tokens in ``tok_list`` (all when it is None).  ``sink``: one float per head whose
     exponential joins the denominator (a score that has no key and no value)."""
@@ -707,8 +735,8 @@ def attention_rowwise(q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, 
     _call("ps_attention_rowwise", q.data_ptr(), q_stride, k_pool.data_ptr(), v_pool.data_ptr(),
           out.data_ptr(), out_stride, _ptr(tok_list), tok_item.data_ptr(), tok_pos.data_ptr(),
           tables.data_ptr(), tables.shape[1], count, heads, kv_heads, head_dim, page_size, pages,
-          float(scale), int(window), sink, *_check_gate(gate, q.shape[0], heads), dtype_code(q.dtype),
-          _stream())
+          float(scale), int(window), sink, *_check_gate(gate, q.shape[0], heads), _check_cap(softcap),
+          dtype_code(q.dtype), _stream())
     return out
 
 
@@ -720,7 +748,7 @@ def decode_keys_per_block(head_dim: int, waves: int = 4) -> int:
 
 
 def attention_decode(q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, scale, splits,
-                     partial=None, window=0, tok_list=None, waves=4, sink=None, gate=None):
+                     partial=None, window=0, tok_list=None, waves=4, sink=None, gate=None, softcap=0.0):
     """The same result as ``attention_rowwise`` by the split-KV kernel; ``partial`` is float
     scratch of ``count * heads * splits * (head_dim + 2)`` values when ``splits > 1``.
     ``tok_item=None`` says that token t is item t (row t of ``tables``), as in a step of single
@@ -738,7 +766,7 @@ def attention_decode(q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, s
           _ptr(tok_list), _ptr(tok_item), tok_pos.data_ptr(), tables.data_ptr(),
           tables.shape[1], count, heads, kv_heads, head_dim, page_size, pages, float(scale),
           int(window), int(splits), int(waves), _check_sink(sink, heads),
-          *_check_gate(gate, q.shape[0], heads), dtype_code(q.dtype), _stream())
+          *_check_gate(gate, q.shape[0], heads), _check_cap(softcap), dtype_code(q.dtype), _stream())
     return out
 
 
@@ -757,7 +785,7 @@ def merge_linear_supported(dtype, tokens, head_dim, packed) -> bool:
 
 
 def attention_decode_partial(q, k_pool, v_pool, partial, tok_item, tok_pos, tables, heads, scale, splits,
-                             window=0, tok_list=None, waves=4, sink=None):
+                             window=0, tok_list=None, waves=4, sink=None, softcap=0.0):
     """The per-range records of decode attention only (``partial``: float scratch of
     ``count * heads * splits * (head_dim + 2)`` values); ``attention_merge_linear`` merges them.
     ``tok_item=None``: token t is item t, as for ``attention_decode``."""
@@ -781,7 +809,7 @@ def attention_decode_partial(q, k_pool, v_pool, partial, tok_item, tok_pos, tabl
           partial.data_ptr(), partial.numel(), _ptr(tok_list), _ptr(tok_item), tok_pos.data_ptr(),
           tables.data_ptr(), tables.shape[1], count, heads, kv_heads, head_dim, page_size, pages,
           float(scale), int(window), int(splits), int(waves), _check_sink(sink, heads),
-          dtype_code(q.dtype), _stream())
+          _check_cap(softcap), dtype_code(q.dtype), _stream())
     return count
 
 
@@ -887,7 +915,7 @@ def prefill_large_tile_pays(heads, head_dim, large_tiles, max_kv_len=0) -> bool:
 
 def attention_prefill(q, k_pool, v_pool, out, tile_item, tile_q0, cu_tokens, kv_lens, tables,
                       heads, scale, window=0, max_kv_len=0, query_tile=PREFILL_TILE, memo=None,
-                      shared=None, sink=None, gate=None):
+                      shared=None, sink=None, gate=None, softcap=0.0):
     """Attention of items with several tokens, ``query_tile`` (64, 32 or 128) queries per block,
     on the matrix cores.  Blocks start in the order of the tile list, which is cut for that size:
     the tiles that see the most keys belong first.
@@ -898,7 +926,7 @@ def attention_prefill(q, k_pool, v_pool, out, tile_item, tile_q0, cu_tokens, kv_
         step_key = ("prefill", q.data_ptr(), q.shape[0], out.data_ptr(),
                     tile_item.data_ptr(), tile_item.numel(), tile_q0.data_ptr(), cu_tokens.data_ptr(),
                     cu_tokens.numel(), kv_lens.data_ptr(), tables.data_ptr(), tables.shape[1], heads, scale,
-                    window, max_kv_len, query_tile, _ptr(sink), _ptr(gate))
+                    window, max_kv_len, query_tile, _ptr(sink), _ptr(gate), softcap)
         key = step_key + (k_pool.data_ptr(), v_pool.data_ptr())
         kept = memo.get(key) or _sibling_call(memo, shared, key, step_key, k_pool, v_pool)
         if kept is not None:
@@ -929,7 +957,7 @@ def attention_prefill(q, k_pool, v_pool, out, tile_item, tile_q0, cu_tokens, kv_
                 cu_tokens.data_ptr(), kv_lens.data_ptr(), tables.data_ptr(), tables.shape[1], heads,
                 kv_heads, head_dim, page_size, pages, float(scale), int(window), int(max_kv_len),
                 int(query_tile), _check_sink(sink, heads), *_check_gate(gate, q.shape[0], heads),
-                dtype_code(q.dtype)),
+                _check_cap(softcap), dtype_code(q.dtype)),
                shared, step_key, (kv_heads, head_dim, page_size, pages, q.dtype))
     return out
 
@@ -944,7 +972,7 @@ _TILED_F32_CHECKED = False
 
 
 def attention_tiled_f32(q, k_pool, v_pool, out, tile_item, tile_q0, cu_tokens, kv_lens, tables, heads,
-                        scale, window=0, sink=None, gate=None):
+                        scale, window=0, sink=None, gate=None, softcap=0.0):
     """Attention of items with several tokens in true 32-bit, ``PREFILL_TILE`` queries per
     block: keys and values pass through LDS once per tile of queries instead of once per query
     (``attention_rowwise``), scores and sums are plain float arithmetic.  The tile list is the
@@ -980,7 +1008,7 @@ def attention_tiled_f32(q, k_pool, v_pool, out, tile_item, tile_q0, cu_tokens, k
           out.data_ptr(), out_stride, tile_item.data_ptr(), tile_q0.data_ptr(), tiles,
           cu_tokens.data_ptr(), kv_lens.data_ptr(), tables.data_ptr(), tables.shape[1], heads,
           kv_heads, head_dim, page_size, pages, float(scale), int(window), _check_sink(sink, heads),
-          *_check_gate(gate, q.shape[0], heads), _stream())
+          *_check_gate(gate, q.shape[0], heads), _check_cap(softcap), _stream())
     return out
 
 
@@ -1032,7 +1060,7 @@ def _sibling_call(memo, shared, key, step_key, k_pool, v_pool):
 
 def attention_mixed(q, k_pool, v_pool, out, tok_list, tok_item, positions, tile_item, tile_q0,
                     cu_tokens, kv_lens, tables, heads, scale, window=0, memo=None, shared=None,
-                    sink=None, gate=None):
+                    sink=None, gate=None, softcap=0.0):
     """The attention of a step that mixes decoded tokens with prompt portions, in one launch:
     the tokens listed in ``tok_list`` (the step's one-token items) as ``attention_decode`` with
     one range of keys computes them, the tiles of 64 queries listed in ``tile_item`` /
@@ -1048,7 +1076,7 @@ def attention_mixed(q, k_pool, v_pool, out, tok_list, tok_item, positions, tile_
                     tok_list.data_ptr(), tok_list.numel(), tok_item.data_ptr(), positions.data_ptr(),
                     tile_item.data_ptr(), tile_item.numel(), tile_q0.data_ptr(), cu_tokens.data_ptr(),
                     cu_tokens.numel(), kv_lens.data_ptr(), tables.data_ptr(), tables.shape[1], heads, scale, window,
-                    _ptr(sink), _ptr(gate))
+                    _ptr(sink), _ptr(gate), softcap)
         key = step_key + (k_pool.data_ptr(), v_pool.data_ptr())
         kept = memo.get(key) or _sibling_call(memo, shared, key, step_key, k_pool, v_pool)
         if kept is not None:
@@ -1082,7 +1110,8 @@ def attention_mixed(q, k_pool, v_pool, out, tok_list, tok_item, positions, tile_
                 positions.data_ptr(), tile_item.data_ptr(), tile_q0.data_ptr(), tiles,
                 cu_tokens.data_ptr(), kv_lens.data_ptr(), tables.data_ptr(), tables.shape[1], heads,
                 kv_heads, head_dim, page_size, pages, float(scale), int(window),
-                _check_sink(sink, heads), *_check_gate(gate, q.shape[0], heads), dtype_code(q.dtype)),
+                _check_sink(sink, heads), *_check_gate(gate, q.shape[0], heads), _check_cap(softcap),
+                dtype_code(q.dtype)),
                shared, step_key, (kv_heads, head_dim, page_size, pages, q.dtype))
     return out
 
@@ -1189,6 +1218,67 @@ def attention_prepare(proj, columns, q_out, k_pool, v_pool, tok_item, tok_pos, t
           int(rot_dims), _ptr(v_first), _ptr(v_lambda), int(v_mode), tok_item.data_ptr(),
           tok_pos.data_ptr(), tables.data_ptr(), tables.shape[1], tokens, heads, kv_heads, key_dim,
           value_dim, cache_dim, page_size, pages, dtype_code(q_out.dtype), _stream())
+
+
+def attention_prepare_heads(proj, columns, q_out, k_pool, v_pool, tok_item, tok_pos, tables, heads,
+                            key_dim, value_dim, freqs=None, rot_dims=0, halves=True, magnitude=1.0,
+                            head_norm=False, eps=1e-6):
+    """``attention_prepare`` for layers that treat every head on its own: rotation of the first
+    ``rot_dims`` dimensions of each head (``halves``: dimension i with i + rot_dims / 2, else 2i
+    with 2i + 1; cosine and sine times ``magnitude``), then ``head_norm``: each head divided by its
+    root mean square over ``key_dim`` (no weight).  ``columns = (q_col, k_col, v_col)``; the value
+    columns are stored as projected and may be the key columns."""
+    _check(proj, "proj", torch.float32, 2)
+    _check(q_out, "q_out", ndim=2)
+    pages, kv_heads, page_size, cache_dim = _check_pools(k_pool, v_pool, q_out.dtype)
+    tokens = proj.shape[0]
+    q_col, k_col, v_col = (int(c) for c in columns)
+    ld = _rows(proj, "proj")
+    if max(q_col + heads * key_dim, k_col + kv_heads * key_dim, v_col + kv_heads * value_dim) > proj.shape[1]:
+        raise KernelError("attention_prepare_heads: the projection's rows are too short for its columns")
+    if q_out.shape[0] < tokens or q_out.shape[1] != heads * cache_dim:
+        raise KernelError(f"attention_prepare_heads: q_out must be [>= {tokens}, {heads} x {cache_dim}]")
+    if cache_dim < max(key_dim, value_dim) or cache_dim > 256:
+        raise KernelError(f"attention_prepare_heads: cached heads of {cache_dim} must hold keys of "
+                          f"{key_dim} and values of {value_dim}, up to 256")
+    _check_step_index(tok_item, tok_pos, tables, tokens)
+    if rot_dims:
+        _float_vector(freqs, "freqs", rot_dims // 2)
+    _call("ps_attention_prepare_heads", proj.data_ptr(), ld, q_col, k_col, v_col, q_out.data_ptr(),
+          _rows(q_out, "q_out"), k_pool.data_ptr(), v_pool.data_ptr(), _ptr(freqs), int(rot_dims),
+          1 if halves else 0, float(magnitude), 1 if head_norm else 0, float(eps), tok_item.data_ptr(),
+          tok_pos.data_ptr(), tables.data_ptr(), tables.shape[1], tokens, heads, kv_heads, key_dim,
+          value_dim, cache_dim, page_size, pages, dtype_code(q_out.dtype), _stream())
+
+
+def latent_prepare(proj, q_col, kv_col, q_out, k_pool, gamma, eps, tok_item, tok_pos, tables, heads,
+                   dim, rank, freqs=None, rot_dims=0, halves=True, magnitude=1.0):
+    """Latent attention between projection and attention: the token's cached row becomes
+    ``[rms_norm(latent) * gamma | rotated key part | zeros]`` and every head's query row gets its
+    rotated part at ``rank .. rank + rot_dims - 1`` and zeros behind (the first ``rank`` places
+    are left to the caller).  ``proj``: per head ``[dim | rot_dims]`` from ``q_col`` on, ``[rank |
+    rot_dims]`` from ``kv_col`` on.  ``k_pool [pages, 1, page, cache_dim]``."""
+    _check(proj, "proj", torch.float32, 2)
+    _check(q_out, "q_out", ndim=2)
+    _check(k_pool, "k_pool", q_out.dtype, 4)
+    pages, kv_heads, page_size, cache_dim = k_pool.shape
+    tokens = proj.shape[0]
+    if kv_heads != 1 or not k_pool.is_contiguous() or cache_dim < rank + rot_dims:
+        raise KernelError(f"latent_prepare: the pool {tuple(k_pool.shape)} must hold one row of at "
+                          f"least {rank + rot_dims} per token")
+    if max(q_col + heads * (dim + rot_dims), kv_col + rank + rot_dims) > proj.shape[1]:
+        raise KernelError("latent_prepare: the projection's rows are too short for its columns")
+    if q_out.shape[0] < tokens or q_out.shape[1] != heads * cache_dim:
+        raise KernelError(f"latent_prepare: q_out must be [>= {tokens}, {heads} x {cache_dim}]")
+    _float_vector(gamma, "gamma", rank)
+    _check_step_index(tok_item, tok_pos, tables, tokens)
+    if rot_dims:
+        _float_vector(freqs, "freqs", rot_dims // 2)
+    _call("ps_latent_prepare", proj.data_ptr(), _rows(proj, "proj"), int(q_col), int(kv_col),
+          q_out.data_ptr(), _rows(q_out, "q_out"), k_pool.data_ptr(), gamma.data_ptr(), float(eps),
+          _ptr(freqs), int(rot_dims), 1 if halves else 0, float(magnitude), tok_item.data_ptr(),
+          tok_pos.data_ptr(), tables.data_ptr(), tables.shape[1], tokens, heads, int(dim), int(rank),
+          cache_dim, page_size, pages, dtype_code(q_out.dtype), _stream())
 
 
 def head_gate(context, gate, heads, head_dim):
@@ -1311,10 +1401,11 @@ def _scan_state(state, channels, states, taps, what):
                           f"{states + taps - 1}]")
 
 
-def conv_silu(proj, u_col, weight, bias, state, states, x, tok_item, cu_tokens, slots):
+def conv_silu(proj, u_col, weight, bias, state, states, x, tok_item, cu_tokens, slots, activation=True):
     """``x[t, c] = silu(bias[c] + sum_j weight[c, j] u[t - taps + 1 + j, c])`` with the raw inputs
     ``u = proj[:, u_col:u_col + channels]`` of the step and, before the step's first token of an
-    item, the inputs that the item's slot kept (``state[slot, c, states:]``, oldest first)."""
+    item, the inputs that the item's slot kept (``state[slot, c, states:]``, oldest first).
+    ``activation=False``: the plain convolution, without the silu; ``x`` may be float."""
     _check(proj, "proj", torch.float32, 2)
     _check(weight, "weight", torch.float32, 2)
     tokens = proj.shape[0]
@@ -1333,7 +1424,68 @@ def conv_silu(proj, u_col, weight, bias, state, states, x, tok_item, cu_tokens, 
     _step_items(cu_tokens, slots, "conv_silu")
     _call("ps_conv_silu", proj.data_ptr(), _rows(proj, "proj"), u_col, weight.data_ptr(), _ptr(bias),
           state.data_ptr(), states, x.data_ptr(), tok_item.data_ptr(), cu_tokens.data_ptr(),
-          slots.data_ptr(), tokens, channels, taps, dtype_code(x.dtype), _stream())
+          slots.data_ptr(), tokens, channels, taps, 1 if activation else 0, dtype_code(x.dtype),
+          _stream())
+
+
+def lru_scan(proj, y_col, x_col, u, gates, block, lam, decay_scale, state, out, cu_tokens, slots, taps):
+    """The gated linear recurrence with one state per channel, per item and token after token:
+    ``a = exp(-decay_scale * sigmoid(gr[t, c]) * softplus(lam[c]))``, ``S = a S + sqrt(1 - a^2)
+    sigmoid(gi[t, c]) u[t, c]``, ``out[t, c] = S * gelu_tanh(proj[t, y_col + c])``; a row of
+    ``gates`` holds, for every run of ``block`` channels, their ``gr`` and then their ``gi``.
+    ``state [slots, channels, taps]``: S, then the channel's last ``taps - 1`` raw inputs of the
+    convolution (``proj[:, x_col + c]``), which this launch also keeps up to date."""
+    _check(proj, "proj", torch.float32, 2)
+    tokens = proj.shape[0]
+    channels = lam.numel()
+    _float_rows(u, "u", tokens, channels)
+    _float_rows(gates, "gates", tokens, 2 * channels)
+    _float_vector(lam, "lam", channels)
+    _scan_state(state, channels, 1, taps, "lru_scan")
+    _check(out, "out", ndim=2)
+    if out.shape[0] < tokens or out.shape[1] != channels or not out.is_contiguous():
+        raise KernelError("lru_scan: out must be contiguous [>= tokens, channels]")
+    if max(y_col, x_col) + channels > proj.shape[1] or min(y_col, x_col) < 0:
+        raise KernelError("lru_scan: the projection's rows are too short for its channels")
+    items = _step_items(cu_tokens, slots, "lru_scan")
+    _call("ps_lru_scan", proj.data_ptr(), _rows(proj, "proj"), int(y_col), int(x_col), u.data_ptr(),
+          gates.data_ptr(), int(block), lam.data_ptr(), float(decay_scale), state.data_ptr(), out.data_ptr(),
+          cu_tokens.data_ptr(), slots.data_ptr(), items, tokens, channels, int(taps),
+          dtype_code(out.dtype), _stream())
+
+
+def block_linear(x, x_step, w, bias, out, out_step, gate=None, k=None):
+    """A product with a block-diagonal matrix.  ``w [blocks, n, kw]`` (stored ``[out, in]``);
+    block ``b`` reads the ``k`` (default ``kw``) columns of ``x`` from ``b * x_step`` on and
+    writes the ``n`` columns of ``out`` from ``b * out_step`` on, plus ``bias[b * n + j]``, times
+    ``sigmoid(gate[t, b * n + j])`` where ``gate`` (float) is given.  ``x`` and ``out`` may be float
+    or of the matrices' type (a float matrix takes and gives float rows)."""
+    _check(x, "x", ndim=2)
+    _check(w, "w", ndim=3)
+    _check(out, "out", ndim=2)
+    blocks, n, kw = w.shape
+    k = kw if k is None else int(k)
+    if k != kw or not w.is_contiguous():
+        raise KernelError(f"block_linear: w {tuple(w.shape)} must be contiguous [blocks, n, {k}]")
+    tokens = x.shape[0]
+    if out.shape[0] < tokens:
+        raise KernelError("block_linear: out has too few rows")
+    x_ld, out_ld = _rows(x, "x"), _rows(out, "out")
+    if x.shape[1] < (blocks - 1) * x_step + k or out.shape[1] < (blocks - 1) * out_step + n:
+        raise KernelError(f"block_linear: rows of {x.shape[1]} / {out.shape[1]} do not hold {blocks} "
+                          f"blocks of {k} inputs ({x_step} apart) / {n} outputs ({out_step} apart)")
+    if bias is not None:
+        _float_vector(bias, "bias", blocks * n)
+    gate_ptr, gate_ld = 0, 0
+    if gate is not None:
+        _check(gate, "gate", torch.float32, 2)
+        if gate.shape[0] < tokens or gate.shape[1] != blocks * n:
+            raise KernelError(f"block_linear: gates must be float [>= {tokens}, {blocks * n}]")
+        gate_ptr, gate_ld = gate.data_ptr(), _rows(gate, "gate")
+    _call("ps_block_linear", x.data_ptr(), dtype_code(x.dtype), x_ld, int(x_step), w.data_ptr(),
+          dtype_code(w.dtype), _ptr(bias), out.data_ptr(), dtype_code(out.dtype), out_ld, int(out_step),
+          gate_ptr, gate_ld, blocks, n, k, tokens, _stream())
+    return out
 
 
 def step_size(low, w, bias, dt):
@@ -1420,14 +1572,18 @@ def selective_scan(x, dt, bc, b_col, c_col, proj, u_col, z_col, a_log, skip, sta
 
 def stream_step(h, tokens, width, add=None, bias=None, norm=None, zero=None):
     """One pass over the float stream ``h`` (``[>= tokens, width]``), every piece optional:
-    ``add = (y, factor)``: ``h += factor * y``; ``bias``: a float row added to every token;
+    ``add = (y, factor)``: ``h += factor * y``, or ``add = (y, factor, column_scale)`` with a float
+    per column: ``h += factor * column_scale * y``; ``bias``: a float row added to every token;
     ``norm = (gamma, eps, normed)``: the RMS norm of the new ``h`` times ``gamma`` goes to ``normed``
     (engine dtype); ``zero``: a float ``[tokens, width]`` buffer that is cleared (it may be ``y``)."""
     _float_rows(h, "h", tokens, width)
-    y, factor, gamma, eps, normed, code = None, 0.0, None, 1.0, None, F32
+    y, factor, gamma, eps, normed, code, column_scale = None, 0.0, None, 1.0, None, F32, None
     if add is not None:
-        y, factor = add
+        y, factor = add[0], add[1]
         _float_rows(y, "y", tokens, width)
+        if len(add) > 2 and add[2] is not None:
+            column_scale = add[2]
+            _float_vector(column_scale, "column_scale", width)
     if bias is not None:
         _float_vector(bias, "bias", width)
     if norm is not None:
@@ -1439,7 +1595,7 @@ def stream_step(h, tokens, width, add=None, bias=None, norm=None, zero=None):
         code = dtype_code(normed.dtype)
     if zero is not None:
         _float_rows(zero, "zero", tokens, width)
-    _call("ps_stream_step", h.data_ptr(), _ptr(y), float(factor), _ptr(bias), _ptr(gamma), float(eps),
+    _call("ps_stream_step", h.data_ptr(), _ptr(y), float(factor), _ptr(column_scale), _ptr(bias), _ptr(gamma), float(eps),
           _ptr(normed), _ptr(zero), tokens, width, code, _stream())
 
 

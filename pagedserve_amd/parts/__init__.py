@@ -1,5 +1,5 @@
-from . import (attention, block, connection, embedding, feed_forward, linear_attention, norm,  # noqa: F401
-               position, side_by_side, state_space)  # noqa: F401  (register kinds)
+from . import (attention, block, connection, embedding, feed_forward, latent_attention,  # noqa: F401
+               linear_attention, norm, position, side_by_side, state_space)  # noqa: F401  (register kinds)
 from .base import (CacheView, Embedding, FeedForward, Head, Mixer, Norm, PagedKVSpec, Part,
                    PositionEncoding, SlotStateSpec, StepContext, StepItem, Workspace)
 from .registry import (ARRANGEMENTS, CONNECTIONS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS, POSITIONS, ROLES,

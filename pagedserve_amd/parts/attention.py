@@ -5,6 +5,7 @@ import torch
 from ..ops import kernels
 from ..weights.loader import MATRIX, VECTOR, ParamSpec
 from .base import Mixer, PagedKVSpec, site_memo
+from .position import rotary_frequencies
 from .registry import register_mixer
 
 
@@ -41,6 +42,20 @@ class Attention(Mixer):
       attention kernels do it where they store the output.
     * ``out_bias``: whether the output projection has a bias, where that differs from ``bias``
       (which then speaks for the packed projection alone).
+    * ``rotary_layout``: ``"neighbours"`` (dimension 2i with 2i+1) or ``"halves"`` (dimension i
+      with i + rotary_dims / 2); ``rotary_scaling = (factor, original, fast, slow)`` stretches
+      the frequencies and scales cosine and sine (``parts/position.py: rotary_frequencies``).
+    * ``head_norm``: after the rotation every query and key head is divided by its own root
+      mean square (no weight, ``norm_eps``).
+    * ``values_from_keys``: there is no value projection; the values are the keys as projected,
+      before rotation and norm (the packed product is ``[q | k]``).
+    * ``score_cap``: ``c > 0``: a scaled score ``s`` enters the softmax as ``c tanh(s / c)``.
+    * ``pad_heads``: heads are cached with their size rounded up to a multiple of this (zeros
+      behind), so that a head size which the tiled kernels do not take still runs on them.
+
+    ``rotary_layout="halves"``, ``rotary_scaling``, ``head_norm`` and ``values_from_keys`` go
+    through the launch that treats every head on its own (``kernels.attention_prepare_heads``);
+    that one does not norm over the whole projection or mix values.
     """
 
     graph_safe = True
@@ -61,7 +76,9 @@ class Attention(Mixer):
                  window: int = 0, bias: bool = True, value_dim: int = 0, qk_norm: bool = False,
                  norm_eps: float = 1e-6, rotary_dims: int = 0, rotary_base: float = 10000.0,
                  sink: bool = False, value_mix: str = "none", head_gate: bool = False,
-                 out_bias=None):
+                 out_bias=None, rotary_layout: str = "neighbours", rotary_scaling=None,
+                 head_norm: bool = False, values_from_keys: bool = False, score_cap: float = 0.0,
+                 pad_heads: int = 0):
         if heads % kv_heads != 0:
             raise ValueError(f"heads ({heads}) must be a multiple of kv_heads ({kv_heads})")
         if not 0 < head_dim <= 256:
@@ -90,14 +107,36 @@ class Attention(Mixer):
         self.has_sink = bool(sink)
         self.value_mix = value_mix
         self.head_gate = bool(head_gate)
+        if rotary_layout not in ("neighbours", "halves"):
+            raise ValueError(f"rotary_layout {rotary_layout!r}; known: neighbours, halves")
+        self.rotary_halves = rotary_layout == "halves"
+        self.rotary_scaling = None if rotary_scaling is None else tuple(float(v) for v in rotary_scaling)
+        self.head_norm = bool(head_norm)
+        self.values_from_keys = bool(values_from_keys)
+        self.score_cap = float(score_cap or 0.0)
+        if self.score_cap < 0:
+            raise ValueError("a score cap must be positive (0: none)")
+        if self.values_from_keys and self.value_dim != self.key_dim:
+            raise ValueError("values that are the keys have the keys' head size")
+        # the launch that treats every head on its own
+        self.head_wise = (self.head_norm or self.values_from_keys or self.rotary_scaling is not None
+                          or (self.rotary_halves and self.rotary_dims > 0))
+        if self.head_wise and (self.qk_norm or value_mix != "none"):
+            raise ValueError("a norm over the whole projection and mixed values do not go with "
+                             "rotary halves, scaled frequencies, head norms or values from keys")
         self.prepared = (self.value_dim != self.key_dim or self.qk_norm or self.rotary_dims > 0
-                         or value_mix != "none" or self.head_gate)
+                         or value_mix != "none" or self.head_gate or self.head_wise
+                         or (pad_heads > 1 and head_dim % pad_heads != 0))
         # the head size that the cache and the attention kernels see
         self.head_dim = head_dim
         if self.value_dim != self.key_dim:
             self.head_dim = -(-max(self.key_dim, self.value_dim) // 16) * 16
         elif self.prepared and head_dim % 2:
             self.head_dim = head_dim + 1
+        if pad_heads > 1:
+            self.head_dim = -(-self.head_dim // pad_heads) * pad_heads
+        if self.head_dim > 256:
+            raise ValueError(f"heads of {head_dim} cached {self.head_dim} wide: at most 256")
         self.q_cols = heads * self.head_dim         # columns of the queries and of the context
         self.kv_cols = kv_heads * self.head_dim
         self.sink = None
@@ -110,6 +149,10 @@ class Attention(Mixer):
         q_col = 0
         k_col = q_col + self.heads * self.key_dim
         v_col = k_col + self.kv_heads * self.key_dim
+        if self.values_from_keys:
+            # (no value columns: the key columns are read twice)
+            gate_col = v_col
+            return q_col, k_col, k_col, gate_col, gate_col + (self.heads if self.head_gate else 0)
         gate_col = v_col + self.kv_heads * self.value_dim
         return q_col, k_col, v_col, gate_col, gate_col + (self.heads if self.head_gate else 0)
 
@@ -148,11 +191,12 @@ class Attention(Mixer):
             padded[:, :, :self.value_dim] = self.out_weight.view(self.width, self.heads, self.value_dim)
             self.out_weight = padded.view(self.width, self.q_cols)
         self.freqs = None
+        self.rotary_magnitude = 1.0
         if self.rotary_dims:
             # base^(-2i/dims), worked out in 64-bit and rounded once; the angle is float(p) * f
-            steps = torch.arange(self.rotary_dims // 2, dtype=torch.float64)
-            self.freqs = torch.pow(torch.tensor(self.rotary_base, dtype=torch.float64),
-                                   -2.0 * steps / self.rotary_dims).to(torch.float32).to(self.out_weight.device)
+            freqs, self.rotary_magnitude = rotary_frequencies(self.rotary_dims, self.rotary_base,
+                                                              self.rotary_scaling)
+            self.freqs = freqs.to(torch.float32).to(self.out_weight.device)
         # copies in the layout that the products of few rows (decode steps) read fastest
         self.qkv_packed = kernels.pack_decode_weight(self.qkv_weight)
         self.out_packed = kernels.pack_decode_weight(self.out_weight)
@@ -178,6 +222,13 @@ class Attention(Mixer):
         if self.value_mix != "none":
             v_first = ctx.workspace.first_rows("values_source", self.kv_heads * self.value_dim,
                                                self.dtype, tokens)
+        if self.head_wise:
+            kernels.attention_prepare_heads(
+                proj, (q_col, k_col, v_col), q, cache.k_pool, cache.v_pool, ctx.tok_item, ctx.positions,
+                tables, self.heads, self.key_dim, self.value_dim, freqs=self.freqs,
+                rot_dims=self.rotary_dims, halves=self.rotary_halves, magnitude=self.rotary_magnitude,
+                head_norm=self.head_norm, eps=self.norm_eps)
+            return q, (proj[:, gate_col:gate_col + self.heads] if self.head_gate else None)
         kernels.attention_prepare(
             proj, (q_col, k_col, v_col), q, cache.k_pool, cache.v_pool, ctx.tok_item, ctx.positions,
             tables, self.heads, self.key_dim, self.value_dim, q_gamma=self.q_gamma,
@@ -246,7 +297,7 @@ class Attention(Mixer):
             partial = self._range_records(ctx)
             kernels.attention_decode_partial(q, cache.k_pool, cache.v_pool, partial, ctx.tok_item,
                                              ctx.positions, tables, self.heads, self.scale, splits,
-                                             window=self.window, waves=4, sink=sink)
+                                             window=self.window, waves=4, sink=sink, softcap=self.score_cap)
             kernels.attention_merge_linear(partial, singles, self.heads, self.head_dim, splits,
                                            self.out_weight, self.out_packed, self.out_bias, residual)
             return
@@ -258,7 +309,7 @@ class Attention(Mixer):
                                     ctx.tok_item, ctx.positions, tile_item, tile_q0, ctx.cu_tokens,
                                     ctx.kv_lens, tables, self.heads, self.scale, self.window,
                                     memo=site_memo(self._memo_attention, ctx.workspace),
-                                    shared=ctx.shared_calls, sink=sink, gate=gates)
+                                    shared=ctx.shared_calls, sink=sink, gate=gates, softcap=self.score_cap)
             return self._project_out(context, residual, ctx)
         if singles:
             # one-token items: keys of a request are cut into ranges so that few requests
@@ -280,7 +331,7 @@ class Attention(Mixer):
                                      ctx.positions, tables, self.heads, self.scale, splits,
                                      partial=partial, window=self.window, waves=waves,
                                      tok_list=None if singles == tokens else ctx.single_tokens,
-                                     sink=sink, gate=gates)
+                                     sink=sink, gate=gates, softcap=self.score_cap)
         whole = singles == 0
         if tiled:
             size = kernels.PREFILL_TILE
@@ -298,7 +349,7 @@ class Attention(Mixer):
                                       self.heads, self.scale, self.window,
                                       max_kv_len=ctx.max_kv_len, query_tile=size,
                                       memo=site_memo(self._memo_attention, ctx.workspace),
-                                      shared=ctx.shared_calls, sink=sink, gate=gates)
+                                      shared=ctx.shared_calls, sink=sink, gate=gates, softcap=self.score_cap)
         elif singles < tokens and kernels.tiled_f32_supported(self.dtype, self.head_dim):
             # 32-bit: tiles of queries too, on plain float arithmetic.  The tiles hold the items
             # of several tokens; one-token items that the split-KV kernel did not take (a head
@@ -307,16 +358,16 @@ class Attention(Mixer):
             if tile_item.numel():
                 kernels.attention_tiled_f32(q, cache.k_pool, cache.v_pool, context, tile_item, tile_q0,
                                             ctx.cu_tokens, ctx.kv_lens, tables, self.heads, self.scale,
-                                            self.window, sink=sink, gate=gates)
+                                            self.window, sink=sink, gate=gates, softcap=self.score_cap)
             if not singles and ctx.single_tokens is not None and ctx.single_tokens.numel():
                 kernels.attention_rowwise(q, cache.k_pool, cache.v_pool, context, ctx.tok_item,
                                           ctx.positions, tables, self.heads, self.scale, self.window,
                                           tok_list=None if ctx.single_tokens.numel() == tokens
-                                          else ctx.single_tokens, sink=sink, gate=gates)
+                                          else ctx.single_tokens, sink=sink, gate=gates, softcap=self.score_cap)
         elif singles < tokens:
             kernels.attention_rowwise(q, cache.k_pool, cache.v_pool, context, ctx.tok_item,
                                       ctx.positions, tables, self.heads, self.scale, self.window,
-                                      tok_list=None if whole else ctx.portion_tokens, sink=sink, gate=gates)
+                                      tok_list=None if whole else ctx.portion_tokens, sink=sink, gate=gates, softcap=self.score_cap)
         self._project_out(context, residual, ctx)
 
     def _one_launch(self, singles: int, ctx, tables) -> bool:

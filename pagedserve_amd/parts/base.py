@@ -42,6 +42,9 @@ class PagedKVSpec:
     head_dim: int
     window: int = 0
     value_dim: int = 0     # head size of the cached values where it is not the keys' (0: the same)
+    # True: the values are read from the cached key rows themselves (a latent that is key and
+    # value at once): the entry has one pool, handed out as both
+    values_in_keys: bool = False
 
 
 @dataclass(frozen=True)

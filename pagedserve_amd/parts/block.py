@@ -193,6 +193,73 @@ class ParallelScaledBlock:
             kernels.stream_step(h, ctx.tokens, self.width, add=add, zero=add[0])
 
 
+@register_arrangement("pre_norm_scaled")
+class PreNormScaledBlock:
+    """``h += scale1 * mixer(norm1(h))`` then ``h += scale2 * feed_forward(norm2(h))`` with a
+    learned factor per column on each sublayer's result (``parts/connection.py: column_scale``).
+    A sublayer adds into a float row ``y`` per token; one launch folds ``scale * y`` of the
+    sublayer before into the stream, norms for the next one and clears ``y``
+    (``kernels.stream_step``).  A block's last sum is left to the next block's first launch, or
+    to ``finish``."""
+
+    roles = {"norm1": "norm", "mixer": "mixer", "scale1": "connection",
+             "norm2": "norm", "feed_forward": "feed_forward", "scale2": "connection"}
+    takes_stream_write = True
+
+    def __init__(self, width, dtype, parts):
+        self.width = width
+        self.dtype = dtype
+        self._parts = dict(parts)
+        self.mixer = parts["mixer"]
+        self.sublayers = [(parts["norm1"], self.mixer, parts["scale1"])]
+        if "feed_forward" in parts:
+            self.sublayers.append((parts["norm2"], parts["feed_forward"], parts["scale2"]))
+        for norm, _, _ in self.sublayers:
+            if not hasattr(norm, "gamma_eps"):
+                raise ValueError("a scaled pre-norm block needs RMS norms without a shift")
+
+    @property
+    def graph_safe(self):
+        return all(getattr(part, "graph_safe", False) for part in self._parts.values())
+
+    def parts(self):
+        return dict(self._parts)
+
+    def forward(self, h, ctx, cache):
+        tokens = ctx.tokens
+        normed = ctx.workspace.first_rows("normed", self.width, self.dtype, tokens)
+        # (made cleared; every launch that folds it into the stream clears it again)
+        ctx.workspace.rows("sublayer_sum", self.width, torch.float32, cleared=True)
+        y = ctx.workspace.first_rows("sublayer_sum", self.width, torch.float32, tokens)
+        if ctx.extra is None:
+            ctx.extra = {}
+        add = ctx.extra.pop(_SCALED_ADD, None)
+        for norm, part, scale in self.sublayers:
+            gamma, eps = norm.gamma_eps()
+            kernels.stream_step(h, tokens, self.width, add=add, norm=(gamma, eps, normed),
+                                zero=None if add is None else add[0])
+            if part is self.mixer:
+                part.forward(normed, y, ctx, cache)
+            else:
+                part.forward(normed, y, ctx)
+            add = (y, 1.0, scale.weight)
+        ctx.extra[_SCALED_ADD] = add
+        return h
+
+    def finish(self, h, ctx):
+        """Fold in what the block left (no block follows that would)."""
+        add = ctx.extra.pop(_SCALED_ADD, None) if ctx.extra else None
+        if add is not None:
+            kernels.stream_step(h, ctx.tokens, self.width, add=add, zero=add[0])
+
+
+@register_arrangement("pre_norm_scaled_mixer")
+class PreNormScaledMixerBlock(PreNormScaledBlock):
+    """The same with a mixer only."""
+
+    roles = {"norm1": "norm", "mixer": "mixer", "scale1": "connection"}
+
+
 @register_arrangement("parallel_scaled_mixer")
 class ParallelScaledMixerBlock(ParallelScaledBlock):
     """The same with a mixer only."""

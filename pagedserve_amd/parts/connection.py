@@ -41,3 +41,22 @@ class HyperConnection(Part):
         if pending is None or not pending.rms or pending.beta is not None:
             raise NotImplementedError("a hyper-connected sublayer takes an RMS norm without a shift")
         return (self.in_weights, pending.gamma, pending.eps, normed)
+
+
+@register_connection("column_scale")
+class ColumnScale(Part):
+    """A learned factor per column on what a sublayer adds to the stream ("layer scale"):
+    ``x <- x + weight * sublayer(norm(x))``, element by element.  One parameter, ``weight
+    [width]``, 32-bit."""
+
+    graph_safe = True
+
+    def __init__(self, width: int, dtype):
+        self.width = width
+        self.dtype = dtype
+
+    def parameters(self):
+        return {"weight": ParamSpec((self.width,), VECTOR)}
+
+    def bind(self, tensors):
+        self.weight = tensors["weight"]

@@ -10,7 +10,8 @@ from .registry import register_embedding, register_head
 class TokenLookup(Embedding):
     """``h[t] = scale * table[id[t]] + position_table[pos[t]]`` in float
     (src/model/paged_decoder.py:306-314, where the scale is 1).  A token id may be "what the
-    last step chose for row r", which the kernel reads from the device."""
+    last step chose for row r", which the kernel reads from the device.  ``norm = (gamma, eps)``:
+    the rows are RMS-normed in the same launch (a model that norms its embedding)."""
 
     graph_safe = True
 
@@ -23,9 +24,12 @@ class TokenLookup(Embedding):
     def parameters(self):
         return {"table": ParamSpec((self.vocab_size, self.width), TABLE)}
 
-    def forward(self, ctx, position_table, out):
+    takes_norm = True
+
+    def forward(self, ctx, position_table, out, norm=None):
         return kernels.embed(self.table, position_table, ctx.token_ids, ctx.positions, out,
-                             token_src=ctx.token_src, carried=ctx.carried_tokens, scale=self.scale)
+                             token_src=ctx.token_src, carried=ctx.carried_tokens, scale=self.scale,
+                             norm=norm)
 
 
 @register_head("linear")

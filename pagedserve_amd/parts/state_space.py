@@ -105,3 +105,82 @@ class SelectiveScan(Mixer):
         kernels.linear(y, self.out_weight, None, residual, epilogue="residual",
                        packed=self.out_packed, memo=site_memo(self._memo_out, workspace),
                        shared=ctx.shared_calls)
+
+
+@register_mixer("gated_linear_recurrence")
+class GatedLinearRecurrence(Mixer):
+    """The recurrent block of Griffin with its real-gated linear recurrent unit.  With ``h`` the
+    layer's input, two branches of ``inner`` channels:
+
+        y = gelu_tanh(W_y h + b_y)
+        u = conv(W_x h + b_x)           a causal convolution per channel over ``taps`` inputs, with bias
+        r = sigmoid(A_b u_b + a_b),  i = sigmoid(I_b u_b + i_b)     block by block: the channels in
+                                                                   ``blocks`` runs, a square matrix each
+        a = exp(-decay_scale * r * softplus(lam)),   S_t = a S_(t-1) + sqrt(1 - a^2) * i * u
+        out = W_o (S * y)
+
+    One packed product gives ``[y | x]`` in float, one block-diagonal product the gates of a run
+    ``[r | i]``.  Per request the slot keeps S and, behind it, each channel's last ``taps - 1``
+    inputs of the convolution; both start at zero.  Gates, decays and the state are 32-bit in
+    both engine dtypes (``csrc/linear_recurrence.hip``)."""
+
+    graph_safe = True
+
+    accepts_pending_norm = True
+
+    def __init__(self, width: int, dtype, inner: int, blocks: int, taps: int, decay_scale: float = 8.0):
+        if inner % blocks:
+            raise ValueError(f"{inner} channels do not split into {blocks} equal runs")
+        if not 1 <= taps <= 64:
+            raise ValueError(f"taps {taps} must lie in 1..64")
+        self.width = width
+        self.dtype = dtype
+        self.inner = inner
+        self.blocks = blocks
+        self.block = inner // blocks
+        self.taps = taps
+        self.decay_scale = float(decay_scale)
+        self._memo_in, self._memo_out = {}, {}
+
+    def parameters(self):
+        return {
+            "in.weight": ParamSpec((2 * self.inner, self.width), MATRIX),
+            "in.bias": ParamSpec((2 * self.inner,), VECTOR),
+            "conv.weight": ParamSpec((self.inner, self.taps), VECTOR),
+            "conv.bias": ParamSpec((self.inner,), VECTOR),
+            "gates.weight": ParamSpec((self.blocks, 2 * self.block, self.block), MATRIX),
+            "gates.bias": ParamSpec((self.blocks, 2 * self.block), VECTOR),
+            "lam": ParamSpec((self.inner,), VECTOR),
+            "out.weight": ParamSpec((self.width, self.inner), MATRIX),
+        }
+
+    def bind(self, tensors):
+        for name in self.parameters():
+            setattr(self, name.replace(".", "_"), tensors[name])
+        self.gates_bias = self.gates_bias.reshape(-1)
+        self.in_packed = kernels.pack_decode_weight(self.in_weight)
+        self.out_packed = kernels.pack_decode_weight(self.out_weight)
+        for memo in (self._memo_in, self._memo_out):
+            memo.clear()
+
+    def cache_spec(self):
+        return SlotStateSpec((self.inner, self.taps), torch.float32)
+
+    def forward(self, x, residual, ctx, cache):
+        tokens = ctx.tokens
+        workspace = ctx.workspace
+        inner = self.inner
+        proj = workspace.first_rows("lru_proj", 2 * inner, torch.float32, tokens)
+        kernels.linear(x, self.in_weight, self.in_bias, proj, packed=self.in_packed,
+                       memo=site_memo(self._memo_in, workspace), shared=ctx.shared_calls)
+        u = workspace.first_rows("lru_u", inner, torch.float32, tokens)
+        kernels.conv_silu(proj, inner, self.conv_weight, self.conv_bias, cache.state, 1, u,
+                          ctx.tok_item, ctx.cu_tokens, ctx.slots, activation=False)
+        gates = workspace.first_rows("lru_gates", 2 * inner, torch.float32, tokens)
+        kernels.block_linear(u, self.block, self.gates_weight, self.gates_bias, gates, 2 * self.block)
+        y = workspace.first_rows("lru_y", inner, self.dtype, tokens)
+        kernels.lru_scan(proj, 0, inner, u, gates, self.block, self.lam, self.decay_scale, cache.state,
+                         y, ctx.cu_tokens, ctx.slots, self.taps)
+        kernels.linear(y, self.out_weight, None, residual, epilogue="residual",
+                       packed=self.out_packed, memo=site_memo(self._memo_out, workspace),
+                       shared=ctx.shared_calls)

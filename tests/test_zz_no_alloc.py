@@ -20,7 +20,8 @@ STATIC_ARGS = [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_
                c_int, c_int, c_int, c_void_p]
 BUFFER_ARGS = [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int64,
                c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
-               c_int, c_float, c_int, c_int, c_int, c_void_p, c_void_p, c_int64, c_int, c_void_p]
+               c_int, c_float, c_int, c_int, c_int, c_void_p, c_void_p, c_int64, c_float, c_int,
+               c_void_p]
 STATIC_FLOATS = 2 * 1024 * 1024
 
 
@@ -67,7 +68,7 @@ def _both(lib, case, heads, kv_heads, head_dim, page_size, splits, dtype_code):
     sizes = (tok_item.data_ptr(), tok_pos.data_ptr(), tables.data_ptr(), tables.shape[1], count,
              heads, kv_heads, head_dim, page_size, k_pool.shape[0], head_dim ** -0.5, 0, splits, 4)
     common = sizes + (dtype_code, stream)
-    with_sink = sizes + (None, None, 0, dtype_code, stream)     # (the buffer variant takes a sink and gates; none here)
+    with_sink = sizes + (None, None, 0, 0.0, dtype_code, stream)     # (the buffer variant takes a sink, gates and a score cap; none here)
     got = torch.full_like(q, float("nan"))
     status = lib.ps_attention_decode_static(q.data_ptr(), q.stride(0), k_pool.data_ptr(),
                                             v_pool.data_ptr(), got.data_ptr(), got.stride(0),
