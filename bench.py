@@ -32,6 +32,7 @@ One JSON line is printed:
     python bench.py --kernels [--shape small|medium|xl|all] [--only name,name]
     python bench.py --design kosesun [--sizes small,small_narrow,medium]   Kosesun beside GPT-2 at equal size
     python bench.py --design zetunex [--sizes small,medium,small_many_experts]   Zetunex beside Kosesun at equal size
+    python bench.py --design rezelix [--sizes small,medium,small_wide_heads]     Rezelix beside Zetunex at equal size
 
 ``--kernels`` times every kernel of a decode step (1, 8 and 64 requests over 1,024 keys), of
 the prefill step (2 x 1,024 tokens) and of a mixed step (32 decoded tokens beside a portion of
@@ -556,7 +557,49 @@ ZETUNEX_SIZES = {
     "small_many_experts": (zetunex_shape(768, 12, 12, 4, 64, 3072, 50257, experts=16),
                            kosesun_shape(768, 12, 12, 4, 64, 64, 3072, 50257)),
 }
-DESIGNS = {"kosesun": (("kosesun", "gpt2"), DESIGN_SIZES), "zetunex": (("zetunex", "kosesun"), ZETUNEX_SIZES)}
+
+
+def rezelix_shape(width, layers, heads, kv_heads, dim, ff, vocab, rank=192, rot_dim=64):
+    """A Rezelix configuration of a real model's layer sizes: two recurrent layers (as wide as the
+    model, one gate block per head, four taps), then attention with grouped heads whose values are
+    the keys, then latent attention (a latent of ``rank`` with a rotated part of ``rot_dim``); every
+    layer has a gated feed-forward."""
+    scaling = {"factor": 8.0, "original": 2048, "fast": 32.0, "slow": 1.0}
+    listed = []
+    for index in range(layers):
+        kind = ("rglru", "rglru", "attention", "latent_attention")[index % 4]
+        if kind == "rglru":
+            mixer = {"width": width, "blocks": heads, "conv": 4}
+        elif kind == "attention":
+            mixer = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5,
+                     "softcap": 30.0, "rot": {"dims": dim, "base": 10000.0, "scaling": scaling}}
+        else:
+            mixer = {"heads": heads, "dim": dim, "rot_dim": rot_dim, "vdim": dim, "kv_rank": rank,
+                     "scale": (dim + rot_dim) ** -0.5,
+                     "rot": {"dims": rot_dim, "base": 10000.0, "scaling": scaling}}
+        listed.append({"type": kind, "mixer": mixer, "mlp": {"kind": "dense", "ff": ff}})
+    return {"architecture": "Rezelix", "vocab": vocab, "width": width, "layers": listed, "norm": {"eps": 1e-6}}
+
+
+def _dense_zetunex(width, layers, heads, kv_heads, dim, ff, vocab):
+    """The Zetunex shape with dense feed-forwards only (Rezelix has no experts)."""
+    raw = zetunex_shape(width, layers, heads, kv_heads, dim, ff, vocab)
+    for entry in raw["layers"]:
+        entry["mlp"] = {"kind": "dense", "ff": ff}
+    return raw
+
+
+# name -> (Rezelix configuration, the Zetunex configuration of equal width, depth, heads and inner
+# width, with dense feed-forwards)
+REZELIX_SIZES = {
+    "small": (rezelix_shape(768, 12, 12, 4, 64, 3072, 50257), _dense_zetunex(768, 12, 12, 4, 64, 3072, 50257)),
+    "medium": (rezelix_shape(1024, 24, 16, 4, 64, 4096, 50257), _dense_zetunex(1024, 24, 16, 4, 64, 4096, 50257)),
+    # heads of 128 and a narrow latent
+    "small_wide_heads": (rezelix_shape(768, 12, 6, 2, 128, 3072, 50257, rank=96, rot_dim=32),
+                         _dense_zetunex(768, 12, 6, 2, 128, 3072, 50257)),
+}
+DESIGNS = {"kosesun": (("kosesun", "gpt2"), DESIGN_SIZES), "zetunex": (("zetunex", "kosesun"), ZETUNEX_SIZES),
+           "rezelix": (("rezelix", "zetunex"), REZELIX_SIZES)}
 
 
 def design_comparison(args):
@@ -663,8 +706,8 @@ def main(argv=None):
     parser.add_argument("--rows", default="1,8,64", help="decode batch sizes of --kernels")
     parser.add_argument("--only", help="--kernels: only kernels whose name holds one of these (comma-separated)")
     parser.add_argument("--no-prefill", action="store_true", help="--kernels: decode tables only")
-    parser.add_argument("--design", choices=("kosesun", "zetunex"), default=None,
-                        help="prefill and decode throughput of this design beside GPT-2 at equal size")
+    parser.add_argument("--design", choices=("kosesun", "zetunex", "rezelix"), default=None,
+                        help="prefill and decode throughput of this design beside the closest other one at equal size")
     parser.add_argument("--sizes", default="small,small_narrow,medium", help="--design: which sizes")
     args = parser.parse_args(argv)
     if args.gpus != 1:
