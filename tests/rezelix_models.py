@@ -2,6 +2,7 @@
 constants that differ from each other in every respect, and folders with random weights."""
 
 import json
+import math
 import os
 
 import torch
@@ -149,6 +150,6 @@ def loud_key_model(tmp_path, kind, decay=0.9995):
         up[:, :4, :4] = torch.eye(4) * 2.0
         q.view(2, 20, width)[:, :4, 1] = 1.5
     # the recurrent layer: slow decays, so that what LOUD wrote is still there hundreds of tokens on
-    w["l1.mix.lam"] = torch.full((32,), float(torch.log(torch.expm1(torch.tensor(-torch.log(torch.tensor(decay)) / 8.0)))))
+    w["l1.mix.lam"] = torch.full((32,), math.log(math.expm1(-math.log(decay) / 8.0)))
     folder = os.path.join(str(tmp_path), f"rezelix_loud_{kind}")
     return folder, raw, write_folder(folder, raw, w)
