@@ -12,11 +12,14 @@
 // taps - 1 raw inputs of the short convolution (proj[:, x_col + c], oldest first), which the
 // convolution kernel of selective_scan.hip reads at the next step.
 //
-// The recurrence is linear in S, so a run of tokens acts on S as S -> A S + B.  A block owns 64
-// channels of one item; its SEG x 64 threads cut the item's tokens into runs of L: every thread
+// The recurrence is linear in S, so a run of tokens acts on S as S -> A S + B.  A block owns CH
+// channels of one item; its SEG x CH threads cut the item's tokens into runs of L: every thread
 // works out a and b of its run's tokens and the run's (A, B), the runs' starts follow from the
 // carried state through LDS, and every thread walks its run again from its true start, out of
-// registers.  The dependent chain of an item of n tokens is n / SEG steps long, not n.
+// registers.  The dependent chain of an item of n tokens is n / SEG steps long, not n.  Long
+// portions of few items take 16 channels and 64 runs a block, so that two prompts of a model
+// 768 wide are 96 blocks and not 24 (a wave then reads four tokens' 64 bytes, not one token's
+// 256); many items or many channels fill the chip with 64 channels a block.
 #include <math.h>
 
 #include "common.h"
@@ -40,14 +43,14 @@ struct LruArgs {
 __device__ inline float lru_softplus(float x) { return fmaxf(x, 0.f) + log1pf(expf(-fabsf(x))); }
 __device__ inline float lru_sigmoid(float x) { return 1.0f / (1.0f + expf(-x)); }
 
-template <typename T, int SEG, int L>
-__global__ __launch_bounds__(64 * SEG) void lru_scan_kernel(LruArgs p, T* __restrict__ out) {
-  __shared__ float s_a[SEG][64], s_b[SEG][64];
-  __shared__ float s_carry[64];
+template <typename T, int CH, int SEG, int L>
+__global__ __launch_bounds__(CH * SEG) void lru_scan_kernel(LruArgs p, T* __restrict__ out) {
+  __shared__ float s_a[SEG][CH], s_b[SEG][CH];
+  __shared__ float s_carry[CH];
   const int item = blockIdx.x;
-  const int lane = threadIdx.x & 63;
-  const int seg = threadIdx.x >> 6;
-  const int c = blockIdx.y * 64 + lane;
+  const int lane = threadIdx.x % CH;
+  const int seg = threadIdx.x / CH;
+  const int c = blockIdx.y * CH + lane;
   const bool live = c < p.channels;
   const int cc = live ? c : p.channels - 1;
   const int t0 = p.cu_tokens[item], t1 = p.cu_tokens[item + 1];
@@ -124,14 +127,19 @@ extern "C" int ps_lru_scan(const float* proj, int64_t ld, int y_col, int x_col, 
   hipStream_t s = (hipStream_t)stream;
   const LruArgs p = {proj, ld, y_col, x_col, u, gates, block, lam, decay_scale, state, cu_tokens, slots, channels, taps};
   const dim3 grid(items, (channels + 63) / 64);
-  // decoded tokens and short portions: one wave walks an item; long portions: 16 runs side by side
+  const dim3 narrow_grid(items, (channels + 15) / 16);
+  // decoded tokens and short portions: one wave walks an item; long portions: 16 runs side by
+  // side, or 64 runs of 16 channels where blocks of 64 channels would leave most of the chip idle
   const bool wide = tokens - items >= 64;
-#define PS_LAUNCH_LRU(T)                                                                         \
-  do {                                                                                           \
-    if (wide)                                                                                    \
-      hipLaunchKernelGGL((lru_scan_kernel<T, 16, 8>), grid, dim3(1024), 0, s, p, (T*)out);       \
-    else                                                                                         \
-      hipLaunchKernelGGL((lru_scan_kernel<T, 1, 4>), grid, dim3(64), 0, s, p, (T*)out);          \
+  const bool narrow = wide && (int64_t)grid.x * grid.y < 192;
+#define PS_LAUNCH_LRU(T)                                                                              \
+  do {                                                                                                \
+    if (narrow)                                                                                       \
+      hipLaunchKernelGGL((lru_scan_kernel<T, 16, 64, 4>), narrow_grid, dim3(1024), 0, s, p, (T*)out); \
+    else if (wide)                                                                                    \
+      hipLaunchKernelGGL((lru_scan_kernel<T, 64, 16, 8>), grid, dim3(1024), 0, s, p, (T*)out);        \
+    else                                                                                              \
+      hipLaunchKernelGGL((lru_scan_kernel<T, 64, 1, 4>), grid, dim3(64), 0, s, p, (T*)out);           \
   } while (0)
   if (dtype == PS_F32)
     PS_LAUNCH_LRU(float);
