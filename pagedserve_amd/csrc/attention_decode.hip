@@ -112,6 +112,24 @@ static int launch_decode(const void* q, int64_t q_stride, const void* k_pool, co
   return 0;
 }
 
+// The merge of the ranges' records alone, for kernels of other files that write such records.
+int ps_attention_reduce(const float* partial, void* out, int64_t out_stride, const int* tok_list, int count,
+                        int heads, int head_dim, int splits, const float* gate, int64_t gate_ld, int dtype,
+                        void* stream) {
+  PS_REQUIRE(count > 0 && heads > 0 && heads <= 65535 && splits >= 1 && splits <= 64,
+             "ps_attention_reduce: bad sizes");
+  const AttnExtras extra{nullptr, gate, gate_ld, 0.f};
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == PS_F32)
+    hipLaunchKernelGGL(attention_reduce_kernel<float>, dim3(count, heads), dim3(64), 0, s, partial, (float*)out,
+                       out_stride, tok_list, heads, head_dim, splits, extra);
+  else
+    hipLaunchKernelGGL(attention_reduce_kernel<bf16_t>, dim3(count, heads), dim3(64), 0, s, partial, (bf16_t*)out,
+                       out_stride, tok_list, heads, head_dim, splits, extra);
+  PS_CHECK_LAUNCH("ps_attention_reduce");
+  return 0;
+}
+
 static int check_decode_sizes(const char* who, int count, int heads, int kv_heads, int head_dim,
                               int page_size, int num_pages, int table_width, int window,
                               int splits, int waves, int dtype) {

@@ -157,6 +157,19 @@ int ps_attention_decode(const void* q, int64_t q_stride, const void* k_pool, con
                         int splits, int waves, const float* sink, const float* gate, int64_t gate_ld,
                         float softcap, int dtype, void* stream);
 
+// The same result for bfloat16 layers whose query heads share key/value heads in large groups
+// (one cached row that all heads read): a block takes a token's heads of one group (up to 16)
+// and a range of keys, loads the keys once and serves every head on the matrix cores.  `partial`
+// (count * heads * splits * (head_dim + 2) floats) is needed with one range too; no sink.
+// v_pool may be k_pool.
+int ps_attention_decode_shared(const void* q, int64_t q_stride, const void* k_pool, const void* v_pool,
+                               void* out, int64_t out_stride, float* partial, int64_t partial_floats,
+                               const int* tok_list, const int* tok_item, const int* tok_pos,
+                               const int* tables, int table_width, int count, int heads, int kv_heads,
+                               int head_dim, int page_size, int num_pages, float scale, int window,
+                               int splits, const float* gate, int64_t gate_ld, float softcap,
+                               void* stream);
+
 // Only the records of ps_attention_decode: (unnormalised sum of values [head_dim], maximum in
 // units of log 2, sum) per (token, head, range) at partial[((n * heads + head) * splits + s) *
 // (head_dim + 2)], also with one range; nothing is merged and no output rows are written.

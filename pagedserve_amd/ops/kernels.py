@@ -91,6 +91,10 @@ _SIGNATURES = {
                             c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                             c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_void_p, c_void_p,
                             c_int64, c_float, c_int, c_void_p],
+    "ps_attention_decode_shared": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p,
+                                   c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
+                                   c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_void_p, c_int64,
+                                   c_float, c_void_p],
     "ps_attention_decode_partial": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p,
                                     c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
                                     c_int, c_int, c_float, c_int, c_int, c_int, c_void_p, c_float, c_int,
@@ -767,6 +771,38 @@ def attention_decode(q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, s
           tables.shape[1], count, heads, kv_heads, head_dim, page_size, pages, float(scale),
           int(window), int(splits), int(waves), _check_sink(sink, heads),
           *_check_gate(gate, q.shape[0], heads), _check_cap(softcap), dtype_code(q.dtype), _stream())
+    return out
+
+
+SHARED_DECODE_KEYS = 64       # keys per tile of the kernel below
+SHARED_DECODE_HEADS = 16      # heads of a group that one block serves
+
+
+def shared_decode_supported(dtype, heads, kv_heads, head_dim, sink=None) -> bool:
+    """Whether ``attention_decode_shared`` takes a layer and pays: bfloat16, no sink, and at least
+    six query heads to a key/value head (with fewer, a block's tile of 16 heads is mostly empty
+    and the kernel per head is as fast)."""
+    return (dtype == torch.bfloat16 and sink is None and head_dim % 8 == 0 and 0 < head_dim <= 256
+            and heads % kv_heads == 0 and heads // kv_heads >= 6)
+
+
+def attention_decode_shared(q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, scale, splits, partial,
+                            window=0, tok_list=None, gate=None, softcap=0.0):
+    """``attention_decode`` by blocks that load a tile of keys once for all heads of a group (up
+    to 16) and work on the matrix cores; ``v_pool`` may be ``k_pool``.  ``partial``: float scratch of
+    ``count * heads * splits * (head_dim + 2)`` values, also with one range."""
+    pages, kv_heads, page_size, head_dim, q_stride, out_stride, count = _attention_args(
+        q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, tok_list, direct_items=True)
+    if q.dtype != torch.bfloat16:
+        raise KernelError("attention_decode_shared: bfloat16 only")
+    _check(partial, "partial", torch.float32)
+    if not partial.is_contiguous():
+        raise KernelError("attention_decode_shared: scratch must be contiguous")
+    _call("ps_attention_decode_shared", q.data_ptr(), q_stride, k_pool.data_ptr(), v_pool.data_ptr(),
+          out.data_ptr(), out_stride, partial.data_ptr(), partial.numel(), _ptr(tok_list), _ptr(tok_item),
+          tok_pos.data_ptr(), tables.data_ptr(), tables.shape[1], count, heads, kv_heads, head_dim,
+          page_size, pages, float(scale), int(window), int(splits), *_check_gate(gate, q.shape[0], heads),
+          _check_cap(softcap), _stream())
     return out
 
 

@@ -311,7 +311,16 @@ class Attention(Mixer):
                                     memo=site_memo(self._memo_attention, ctx.workspace),
                                     shared=ctx.shared_calls, sink=sink, gate=gates, softcap=self.score_cap)
             return self._project_out(context, residual, ctx)
-        if singles:
+        if singles and kernels.shared_decode_supported(self.dtype, self.heads, self.kv_heads, self.head_dim, sink):
+            # many heads to a key/value head: blocks that load a tile of keys once for all of them
+            kernels.attention_decode_shared(q, cache.k_pool, cache.v_pool, context,
+                                            None if singles == tokens else ctx.tok_item, ctx.positions,
+                                            tables, self.heads, self.scale,
+                                            self._shared_splits(singles, ctx.max_kv_len),
+                                            self._range_records(ctx), window=self.window,
+                                            tok_list=None if singles == tokens else ctx.single_tokens,
+                                            gate=gates, softcap=self.score_cap)
+        elif singles:
             # one-token items: keys of a request are cut into ranges so that few requests
             # still fill the chip
             splits, waves = self._splits(singles, ctx.max_kv_len)
@@ -429,6 +438,19 @@ class Attention(Mixer):
         if tiles * pairs * splits * (self.head_dim + 2) * 4 > 12_000_000:
             return 0
         return splits
+
+    def _shared_splits(self, count: int, max_kv_len: int) -> int:
+        """Ranges per request of the decode kernel whose blocks serve a group's heads together:
+        about two blocks per compute unit, no range shorter than a tile of keys, and never more
+        records than the scratch holds (six per unit beside one per token and head)."""
+        visible = max_kv_len if self.window <= 0 else min(max_kv_len, self.window)
+        units = kernels.compute_units()
+        group = self.heads // self.kv_heads
+        blocks = count * self.kv_heads * -(-group // kernels.SHARED_DECODE_HEADS)
+        wanted = -(-2 * units // blocks)
+        most = -(-visible // kernels.SHARED_DECODE_KEYS)
+        room = 1 + 6 * units // (count * self.heads)
+        return max(1, min(wanted, most, room, 64))
 
     def _splits(self, count: int, max_kv_len: int):
         """(ranges per request, waves per block) of the decode kernel, by the number of (token,

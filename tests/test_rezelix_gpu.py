@@ -324,6 +324,75 @@ def test_latent_row_normed_rotated_and_stored_and_the_queries_rotated_part(dtype
     assert int((~untouched).sum()) == len(written)
 
 
+def _scores_capped(scores, cap):
+    return scores if not cap else cap * torch.tanh(scores / cap)
+
+
+@pytest.mark.parametrize("heads,kv_heads,dim,same,cap,window", [(12, 1, 256, True, 0.0, 0), (6, 1, 80, True, 0.0, 0),
+                                                              (16, 2, 64, False, 5.0, 0), (40, 2, 32, False, 0.0, 0),
+                                                              (7, 1, 128, False, 3.0, 37), (12, 2, 16, True, 0.0, 0)])
+def test_single_queries_whose_heads_share_a_tile_of_keys(heads, kv_heads, dim, same, cap, window):
+    """Requests of unequal length (one key, a tile's last and first key, hundreds) over pages in
+    any order, every number of ranges; one loud key far back that takes most of a head's weight."""
+    kernels = _kernels()
+    g = torch.Generator().manual_seed(heads * dim)
+    page_size, lengths = 8, [1, 64, 65, 300, 7, 129]
+    count = len(lengths)
+    width = max(-(-n // page_size) for n in lengths)
+    pages = count * width
+    order = torch.randperm(pages, generator=g).tolist()
+    tables = torch.full((count, width), -1, dtype=torch.int32)
+    for n, length in enumerate(lengths):
+        for logical in range(-(-length // page_size)):
+            tables[n, logical] = order.pop()
+    k_pool = torch.randn((pages, kv_heads, page_size, dim), generator=g).to(torch.bfloat16)
+    v_pool = k_pool if same else torch.randn((pages, kv_heads, page_size, dim), generator=g).to(torch.bfloat16)
+    q = torch.randn((count, heads * dim), generator=g).to(torch.bfloat16)
+    # request 3: head 1 points along its third key, long
+    loud_page, loud_place = int(tables[3, 0]), 2
+    q.view(count, heads, dim)[3, 1] = (k_pool[loud_page, 1 // (heads // kv_heads), loud_place].float() * 3).to(torch.bfloat16)
+    gate = torch.randn((count, heads), generator=g)
+    scale = dim ** -0.5
+    expected = torch.zeros((count, heads, dim), dtype=F64)
+    for n, length in enumerate(lengths):
+        first = max(0, length - window) if window else 0
+        rows = [(int(tables[n, p // page_size]), p % page_size) for p in range(first, length)]
+        for h in range(heads):
+            kv = h // (heads // kv_heads)
+            keys = torch.stack([k_pool[page, kv, place] for page, place in rows]).double()
+            values = torch.stack([v_pool[page, kv, place] for page, place in rows]).double()
+            scores = _scores_capped((keys @ q.view(count, heads, dim)[n, h].double()) * scale, cap)
+            weights = torch.softmax(scores, 0)
+            if n == 3 and h == 1 and not window and not cap:
+                assert float(weights[2]) > 0.5
+            expected[n, h] = (weights @ values) * torch.sigmoid(gate[n, h].double())
+    dk = k_pool.cuda()
+    dv = dk if same else v_pool.cuda()
+    positions = _ints([length - 1 for length in lengths])
+    scale_of = float(expected.abs().max())
+    for splits in (1, 2, 3, 5, 64):
+        out = torch.full((count, heads * dim), float("nan"), dtype=torch.bfloat16, device="cuda")
+        partial = torch.full((count * heads * splits * (dim + 2),), float("nan"), device="cuda")
+        for direct in (True, False):
+            kernels.attention_decode_shared(q.cuda(), dk, dv, out, None if direct else _ints(list(range(count))),
+                                            positions, tables.cuda(), heads, scale, splits, partial, window=window,
+                                            gate=gate.cuda(), softcap=cap)
+            got = out.double().cpu().view(count, heads, dim)
+            assert float((got - expected).abs().max()) <= 2e-2 * scale_of, (splits, direct)
+    # a list of some of the tokens: the others' rows stay as they are
+    out = torch.full((count, heads * dim), 7.0, dtype=torch.bfloat16, device="cuda")
+    partial = torch.empty((2 * heads * 2 * (dim + 2),), device="cuda")
+    kernels.attention_decode_shared(q.cuda(), dk, dv, out, _ints(list(range(count))), positions, tables.cuda(),
+                                    heads, scale, 2, partial, window=window, tok_list=_ints([3, 1]),
+                                    gate=gate.cuda(), softcap=cap)
+    got = out.double().cpu().view(count, heads, dim)
+    for n in range(count):
+        if n in (1, 3):
+            assert float((got[n] - expected[n]).abs().max()) <= 2e-2 * scale_of
+        else:
+            assert float((got[n] - 7.0).abs().max()) == 0.0
+
+
 # ---------------------------------------------------------------- whole models
 def _close(rows, reference, dtype):
     """float32: every position within the tolerance.  bfloat16: the bulk of the positions within
