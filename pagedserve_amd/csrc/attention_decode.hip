@@ -43,16 +43,32 @@ __global__ __launch_bounds__(64) void attention_reduce_kernel(
   const float total_l = wave_sum(l_s * weight);
   const float gate = gate_factor(extra, t, head);
   // Every lane takes part in every round, also where head_dim leaves it no dimension: the
-  // weights travel by shuffles, and a shuffle only reads lanes that execute it.
-  for (int d0 = 0; d0 < head_dim; d0 += 64) {
-    const int d = d0 + lane;
-    const bool mine = d < head_dim;
-    const int safe_d = mine ? d : 0;
-    float value = 0.f;
-    for (int s = 0; s < splits; ++s)
-      value = fmaf(src[s * stride + safe_d], __shfl(weight, s, 64), value);
-    if (mine)
-      out[(int64_t)t * out_stride + (int64_t)head * head_dim + d] = from_float<T>(value / total_l * gate);
+  // weights travel by shuffles, and a shuffle only reads lanes that execute it.  A lane owns
+  // dimensions lane, lane + 64, .. (head_dim <= 256: four at most) and asks for eight ranges'
+  // values of all of them at once, so that a merge of many ranges is a few trips to memory and
+  // not one per range and round.
+  float value[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int s0 = 0; s0 < splits; s0 += 8) {
+    float part[4][8];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int d = k * 64 + lane;
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        part[k][j] = (d < head_dim && s0 + j < splits) ? src[(s0 + j) * stride + d] : 0.f;
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float w = __shfl(weight, (s0 + j) & 63, 64);
+#pragma unroll
+      for (int k = 0; k < 4; ++k) value[k] = fmaf(part[k][j], w, value[k]);
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const int d = k * 64 + lane;
+    if (d < head_dim)
+      out[(int64_t)t * out_stride + (int64_t)head * head_dim + d] = from_float<T>(value[k] / total_l * gate);
   }
 }
 
