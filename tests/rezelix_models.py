@@ -78,6 +78,29 @@ MODEL_D = {
                _attention(2, 2, 128, 0.09, None, softcap=8.0, mlp=None),
                _recurrent(200, 5, 2, mlp=_dense(64))],
 }
+# layers of one kind only, and sizes at their ends: a gate block per channel and one block for
+# all, one tap and five, no feed-forward anywhere; one latent head and a latent layer without a
+# rotated part; a latent cached at the widest row the attention kernels take (192 + 64) under
+# eight heads; heads of 8 under one key/value head
+EDGE_MODELS = {
+    "only_recurrent": [_recurrent(24, 24, 1), _recurrent(24, 1, 5, mlp=_dense(16)), _recurrent(64, 2, 3)],
+    "only_latent": [_latent(1, 4, 2, 3, 5, 0.7, _rot(2, 10.0)), _latent(5, 6, 0, 8, 12, 0.3, None, mlp=_dense(24))],
+    "widest_latent": [_latent(8, 64, 64, 32, 192, 0.09, _rot(64, 250000.0, (2.0, 1024, 32.0, 1.0)), mlp=_dense(64)),
+                      _recurrent(32, 4, 3)],
+    "only_attention": [_attention(8, 1, 8, 0.35, _rot(2, 7.0)),
+                       _attention(2, 2, 40, 0.2, _rot(40, 20000.0, (8.0, 2048, 32.0, 1.0)), softcap=20.0, mlp=_dense(48)),
+                       _attention(16, 2, 32, 0.18, _rot(16, 100.0), softcap=2.0)],
+}
+
+
+def edge_folder(tmp_path, which, width=48, vocab=61):
+    """(folder, raw configuration, checkpoint tensors as stored) of one of the models above."""
+    raw = {"architecture": "Rezelix", "vocab": vocab, "width": width, "norm": {"eps": 1e-5},
+           "layers": EDGE_MODELS[which]}
+    folder = os.path.join(str(tmp_path), f"rezelix_edge_{which}")
+    return folder, raw, write_folder(folder, raw, plain_rezelix.random_checkpoint(raw, 5))
+
+
 # name -> (configuration, page size, seed)
 MODELS = {"A": (MODEL_A, 8, 0), "B": (MODEL_B, 16, 1), "C": (MODEL_C, 16, 2), "D": (MODEL_D, 4, 3)}
 

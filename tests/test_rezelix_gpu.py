@@ -454,6 +454,21 @@ def test_model_whole_decoded_in_portions_and_mixed(tmp_path, which, dtype):
             assert any(len(who) > 1 for who in holders.values())
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("which", sorted(rezelix_models.EDGE_MODELS))
+def test_models_of_one_kind_of_layer_and_sizes_at_their_ends(tmp_path, which, dtype):
+    folder, raw, tensors = rezelix_models.edge_folder(tmp_path, which)
+    requests = _requests(raw, (70, 1, 23, 130, 2), 3)
+    reference = _reference(raw, tensors, requests)
+    for name, steps in (("decoded", helpers.trace_tail_decoded(requests, tail=40)),
+                        ("mixed", helpers.trace_mixed(requests, max_live=3))):
+        engine = _engine(folder, dtype, 16, steps, max_requests=3)
+        rows = helpers.replay_in_process(engine, steps)
+        worst, scale, where = helpers.max_error(rows, reference)
+        assert worst <= TOLERANCE[dtype] * scale, (which, name, worst / scale, where)
+        engine.cache.check_invariants()
+
+
 @pytest.mark.parametrize("which", ["A", "D"])
 def test_the_stream_after_every_layer(tmp_path, which):
     """The stream after each layer, read from the engine's workspace while every block folds its
