@@ -564,7 +564,7 @@ def rezelix_shape(width, layers, heads, kv_heads, dim, ff, vocab, rank=192, rot_
     model, one gate block per head, four taps), then attention with grouped heads whose values are
     the keys, then latent attention (a latent of ``rank`` with a rotated part of ``rot_dim``); every
     layer has a gated feed-forward."""
-    scaling = {"factor": 8.0, "original": 2048, "fast": 32.0, "slow": 1.0}
+    scaling = {"factor": 4.0, "original": 4096, "fast": 24.0, "slow": 1.0}
     listed = []
     for index in range(layers):
         kind = ("rglru", "rglru", "attention", "latent_attention")[index % 4]

@@ -66,8 +66,8 @@ MODEL_B = {
 MODEL_C = {
     "architecture": "Rezelix", "vocab": 256, "width": 128, "norm": {"eps": 1e-6},
     "layers": [_recurrent(128, 2, 4, mlp=_dense(256)),
-               _attention(4, 1, 64, 0.125, _rot(64, 10000.0, (8.0, 64, 32.0, 1.0)), softcap=20.0, mlp=_dense(256)),
-               _latent(4, 32, 32, 64, 96, 0.125, _rot(32, 250000.0, (2.0, 32, 16.0, 2.0)), mlp=_dense(128))],
+               _attention(4, 1, 64, 0.125, _rot(64, 10000.0, (6.0, 64, 24.0, 1.0)), softcap=15.0, mlp=_dense(256)),
+               _latent(4, 32, 32, 64, 96, 0.125, _rot(32, 150000.0, (3.0, 32, 16.0, 2.0)), mlp=_dense(128))],
 }
 # wide heads: attention heads of 128 (the decode path that merges key ranges inside the output
 # projection), a latent cached 256 wide (beyond what the 32-bit tiled kernel takes), no rotation
@@ -85,10 +85,10 @@ MODEL_D = {
 EDGE_MODELS = {
     "only_recurrent": [_recurrent(24, 24, 1), _recurrent(24, 1, 5, mlp=_dense(16)), _recurrent(64, 2, 3)],
     "only_latent": [_latent(1, 4, 2, 3, 5, 0.7, _rot(2, 10.0)), _latent(5, 6, 0, 8, 12, 0.3, None, mlp=_dense(24))],
-    "widest_latent": [_latent(8, 64, 64, 32, 192, 0.09, _rot(64, 250000.0, (2.0, 1024, 32.0, 1.0)), mlp=_dense(64)),
+    "widest_latent": [_latent(8, 64, 64, 32, 192, 0.09, _rot(64, 40000.0, (3.0, 256, 20.0, 1.0)), mlp=_dense(64)),
                       _recurrent(32, 4, 3)],
     "only_attention": [_attention(8, 1, 8, 0.35, _rot(2, 7.0)),
-                       _attention(2, 2, 40, 0.2, _rot(40, 20000.0, (8.0, 2048, 32.0, 1.0)), softcap=20.0, mlp=_dense(48)),
+                       _attention(2, 2, 40, 0.2, _rot(40, 30000.0, (6.0, 512, 24.0, 1.5)), softcap=12.0, mlp=_dense(48)),
                        _attention(16, 2, 32, 0.18, _rot(16, 100.0), softcap=2.0)],
 }
 

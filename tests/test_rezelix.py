@@ -138,7 +138,7 @@ def test_one_pool_serves_keys_and_values_of_a_latent_and_counts_once():
 
 
 @pytest.mark.parametrize("dims,base,scaling", [
-    (8, 500.0, (4.0, 16, 8.0, 1.0)), (64, 10000.0, (8.0, 64, 32.0, 1.0)), (32, 250000.0, (2.0, 32, 16.0, 2.0)),
+    (8, 500.0, (4.0, 16, 8.0, 1.0)), (64, 10000.0, (6.0, 64, 24.0, 1.0)), (32, 150000.0, (3.0, 32, 16.0, 2.0)),
     (48, 1000.0, (16.0, 32, 4.0, 1.0)), (12, 10000.0, None), (2, 50.0, (3.0, 100, 2.0, 1.0))])
 def test_stretched_frequencies(dims, base, scaling):
     rot = {"dims": dims, "base": base}

@@ -207,7 +207,7 @@ def test_convolution_without_activation_into_float_rows(channels, taps):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("heads,kv_heads,dim,rot,scaling,norm", [(4, 2, 16, 8, (4.0, 16, 8.0, 1.0), True),
                                                                 (3, 3, 12, 12, None, True),
-                                                                (2, 1, 64, 64, (8.0, 64, 32.0, 1.0), False),
+                                                                (2, 1, 64, 64, (6.0, 64, 24.0, 1.0), False),
                                                                 (2, 2, 128, 0, None, True),
                                                                 (5, 1, 96, 32, (2.0, 40, 16.0, 2.0), True)])
 def test_heads_rotated_in_halves_normed_and_stored_with_the_keys_as_values(dtype, heads, kv_heads, dim, rot,
