@@ -32,6 +32,27 @@ def test_ranges_fit_the_scratch_and_the_kernel(monkeypatch, units):
                         assert count * heads * merged <= 6 * units + count * heads
 
 
+@pytest.mark.parametrize("units", [256, 304, 64])
+def test_ranges_of_the_kernel_for_shared_keys_fit_the_scratch(monkeypatch, units):
+    monkeypatch.setattr(kernels, "compute_units", lambda: units)
+    for heads, kv_heads in ((6, 1), (12, 1), (16, 2), (40, 2), (96, 8), (128, 1)):
+        for window in (0, 300):
+            part = _part(heads, 256, window)
+            part.kv_heads = kv_heads
+            for count in list(range(1, 70)) + [100, 128, 256, 300]:
+                for context in (1, 17, 64, 65, 300, 1024, 4096, 1 << 20):
+                    splits = part._shared_splits(count, context)
+                    assert 1 <= splits <= 64
+                    assert count * heads * splits <= 6 * units + count * heads
+                    # no range without a tile of keys to start at
+                    visible = min(context, window) if window else context
+                    assert splits <= -(-visible // kernels.SHARED_DECODE_KEYS)
+    # 8 requests of 12 heads over one cached row at 1,024 keys: a tile of 64 keys per block
+    part = _part(12, 256)
+    part.kv_heads = 1
+    assert part._shared_splits(8, 1024) == 16 if units == 256 else True
+
+
 def test_documented_cases(monkeypatch):
     monkeypatch.setattr(kernels, "compute_units", lambda: 256)
     part = _part(12)
