@@ -51,7 +51,7 @@ def register_architecture(entry: Architecture) -> Architecture:
 
 def _load_builtin():
     # Importing the module registers it.
-    from ..model import gpt2, kosesun, rezelix, zetunex  # noqa: F401
+    from ..model import gpt2, kosesun, kozapel, rezelix, zetunex  # noqa: F401
 
 
 def find_preset(name: str):

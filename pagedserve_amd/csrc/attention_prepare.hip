@@ -13,6 +13,10 @@
 // the storage type.  Heads are stored `cache_dim` wide (>= the key and the value head size,
 // zeros behind), the one head size that the attention kernels then see for all three.
 // Norm statistics, angles and the mixing are 32-bit.
+//
+// `v_heads` < kv_heads: the projection holds that many value heads and key/value head j caches
+// value head j % v_heads (several maps of keys over the same values).  `store` 0: the layer reads
+// another layer's keys and values; only its queries are prepared.
 #include <math.h>
 
 #include "common.h"
@@ -26,7 +30,8 @@ __global__ __launch_bounds__(1024) void attention_prepare_kernel(
     const float* __restrict__ freqs, int rot_dims, T* __restrict__ v_first,
     const float* __restrict__ v_lambda, int v_mode, const int* __restrict__ tok_item,
     const int* __restrict__ tok_pos, const int* __restrict__ tables, int table_width, int heads,
-    int kv_heads, int key_dim, int value_dim, int cache_dim, int page_size, int num_pages) {
+    int kv_heads, int key_dim, int value_dim, int cache_dim, int page_size, int num_pages,
+    int v_heads, int store) {
   __shared__ float red[2][16];
   __shared__ float s_cos[128], s_sin[128];   // the token's angles, one per rotated pair of a head
   const int t = blockIdx.x;
@@ -43,7 +48,7 @@ __global__ __launch_bounds__(1024) void attention_prepare_kernel(
   // and weights do not wait for the norms: a thread loads its first pair
   // before the block meets for the sums of squares (which the same values feed), so that a
   // step of few tokens makes one trip to memory; further pairs of a thread are read again.
-  const int q_pairs = heads * half, k_pairs = kv_heads * half;
+  const int q_pairs = heads * half, k_pairs = store ? kv_heads * half : 0;
   struct Pair {
     float a, b, wa, wb;
     int head, d0;
@@ -120,12 +125,12 @@ __global__ __launch_bounds__(1024) void attention_prepare_kernel(
     }
   }
   const float lambda = v_mode == 2 ? v_lambda[0] : 0.f;
-  for (int i = threadIdx.x; i < kv_heads * cache_dim; i += blockDim.x) {
+  for (int i = threadIdx.x; i < (store ? kv_heads * cache_dim : 0); i += blockDim.x) {
     const int head = i / cache_dim;
     const int d = i - head * cache_dim;
     float v = 0.f;
     if (d < value_dim) {
-      v = row[v_col + head * value_dim + d];
+      v = row[v_col + (head % v_heads) * value_dim + d];
       const int64_t at = ((int64_t)t * kv_heads + head) * value_dim + d;
       if (v_mode == 1) v_first[at] = from_float<T>(v);
       if (v_mode == 2) v = (1.f - lambda) * v + lambda * to_float<T>(v_first[at]);
@@ -143,7 +148,7 @@ extern "C" int ps_attention_prepare(const float* proj, int64_t ld, int q_col, in
                                     const int* tok_pos, const int* tables, int table_width,
                                     int tokens, int heads, int kv_heads, int key_dim,
                                     int value_dim, int cache_dim, int page_size, int num_pages,
-                                    int dtype, void* stream) {
+                                    int v_heads, int store, int dtype, void* stream) {
   PS_REQUIRE(tokens >= 0 && heads > 0 && kv_heads > 0 && key_dim > 0 && value_dim > 0 &&
                  page_size > 0 && num_pages > 0 && table_width > 0,
              "ps_attention_prepare: bad sizes");
@@ -158,6 +163,9 @@ extern "C" int ps_attention_prepare(const float* proj, int64_t ld, int q_col, in
                  (v_mode != 2 || v_lambda != nullptr),
              "ps_attention_prepare: value mixing needs its buffer and its weight");
   PS_REQUIRE(q_stride >= (int64_t)heads * cache_dim, "ps_attention_prepare: query rows too short");
+  PS_REQUIRE(v_heads >= 1 && v_heads <= kv_heads && kv_heads % v_heads == 0 &&
+                 (v_mode == 0 || v_heads == kv_heads),
+             "ps_attention_prepare: %d value heads under %d key heads", v_heads, kv_heads);
   PS_REQUIRE((q_gamma == nullptr && k_gamma == nullptr) || eps > 0.f, "ps_attention_prepare: eps must be positive");
   PS_REQUIRE(dtype == PS_F32 || dtype == PS_BF16, "ps_attention_prepare: unknown dtype %d", dtype);
   if (tokens == 0) return 0;
@@ -173,13 +181,13 @@ extern "C" int ps_attention_prepare(const float* proj, int64_t ld, int q_col, in
                        k_col, v_col, (float*)q_out, q_stride, (float*)k_pool, (float*)v_pool, q_gamma,
                        k_gamma, eps, freqs, rot_dims, (float*)v_first, v_lambda, v_mode, tok_item,
                        tok_pos, tables, table_width, heads, kv_heads, key_dim, value_dim, cache_dim,
-                       page_size, num_pages);
+                       page_size, num_pages, v_heads, store);
   else
     hipLaunchKernelGGL(attention_prepare_kernel<bf16_t>, dim3(tokens), dim3(threads), 0, s, proj, ld, q_col,
                        k_col, v_col, (bf16_t*)q_out, q_stride, (bf16_t*)k_pool, (bf16_t*)v_pool,
                        q_gamma, k_gamma, eps, freqs, rot_dims, (bf16_t*)v_first, v_lambda, v_mode,
                        tok_item, tok_pos, tables, table_width, heads, kv_heads, key_dim, value_dim,
-                       cache_dim, page_size, num_pages);
+                       cache_dim, page_size, num_pages, v_heads, store);
   PS_CHECK_LAUNCH("ps_attention_prepare");
   return 0;
 }
@@ -366,7 +374,8 @@ extern "C" int ps_attention_prepare_heads(const float* proj, int64_t ld, int q_c
 // holds the weighted latent in its first `rank` places.  A block per token.
 template <typename T>
 __global__ __launch_bounds__(256) void latent_prepare_kernel(
-    const float* __restrict__ proj, int64_t ld, int q_col, int kv_col, T* __restrict__ q_out,
+    const float* __restrict__ proj, int64_t ld, const float* __restrict__ queries, int64_t queries_ld,
+    int q_col, int kv_col, T* __restrict__ q_out,
     int64_t q_stride, T* __restrict__ k_pool, const float* __restrict__ gamma, float eps,
     const float* __restrict__ freqs, int rot_dims, int halves, float magnitude,
     const int* __restrict__ tok_item, const int* __restrict__ tok_pos,
@@ -376,6 +385,7 @@ __global__ __launch_bounds__(256) void latent_prepare_kernel(
   __shared__ float scratch[16];
   const int t = blockIdx.x;
   const float* row = proj + (int64_t)t * ld;
+  const float* q_row = queries + (int64_t)t * queries_ld;
   const int pos = tok_pos[t];
   const int logical = pos / page_size;
   int page = -1;
@@ -402,7 +412,7 @@ __global__ __launch_bounds__(256) void latent_prepare_kernel(
   for (int i = threadIdx.x; i < (heads + 1) * rot_dims; i += blockDim.x) {
     const int vec = i / rot_dims;
     const int d = i - vec * rot_dims;
-    const float* src = vec == 0 ? row + kv_col + rank : row + q_col + (vec - 1) * (dim + rot_dims) + dim;
+    const float* src = vec == 0 ? row + kv_col + rank : q_row + q_col + (vec - 1) * (dim + rot_dims) + dim;
     const RotationPlace place = rotation_place(d, rot_dims, halves != 0);
     const float v = src[d] * s_cos[place.angle] + place.sign * src[place.partner] * s_sin[place.angle];
     if (vec == 0) {
@@ -418,7 +428,8 @@ __global__ __launch_bounds__(256) void latent_prepare_kernel(
   }
 }
 
-extern "C" int ps_latent_prepare(const float* proj, int64_t ld, int q_col, int kv_col, void* q_out,
+extern "C" int ps_latent_prepare(const float* proj, int64_t ld, const float* queries,
+                                 int64_t queries_ld, int q_col, int kv_col, void* q_out,
                                  int64_t q_stride, void* k_pool, const float* gamma, float eps,
                                  const float* freqs, int rot_dims, int halves, float magnitude,
                                  const int* tok_item, const int* tok_pos, const int* tables,
@@ -435,16 +446,18 @@ extern "C" int ps_latent_prepare(const float* proj, int64_t ld, int q_col, int k
              cache_dim, rank, rot_dims);
   PS_REQUIRE(q_stride >= (int64_t)heads * cache_dim, "ps_latent_prepare: query rows too short");
   PS_REQUIRE(gamma != nullptr && eps > 0.f, "ps_latent_prepare: the latent's norm needs its weight and a positive eps");
+  PS_REQUIRE(queries != nullptr && queries_ld >= q_col + (int64_t)heads * (dim + rot_dims),
+             "ps_latent_prepare: the queries' rows are too short");
   PS_REQUIRE(dtype == PS_F32 || dtype == PS_BF16, "ps_latent_prepare: unknown dtype %d", dtype);
   if (tokens == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
   if (dtype == PS_F32)
-    hipLaunchKernelGGL(latent_prepare_kernel<float>, dim3(tokens), dim3(256), 0, s, proj, ld, q_col,
+    hipLaunchKernelGGL(latent_prepare_kernel<float>, dim3(tokens), dim3(256), 0, s, proj, ld, queries, queries_ld, q_col,
                        kv_col, (float*)q_out, q_stride, (float*)k_pool, gamma, eps, freqs, rot_dims,
                        halves, magnitude, tok_item, tok_pos, tables, table_width, heads, dim, rank,
                        cache_dim, page_size, num_pages);
   else
-    hipLaunchKernelGGL(latent_prepare_kernel<bf16_t>, dim3(tokens), dim3(256), 0, s, proj, ld, q_col,
+    hipLaunchKernelGGL(latent_prepare_kernel<bf16_t>, dim3(tokens), dim3(256), 0, s, proj, ld, queries, queries_ld, q_col,
                        kv_col, (bf16_t*)q_out, q_stride, (bf16_t*)k_pool, gamma, eps, freqs, rot_dims,
                        halves, magnitude, tok_item, tok_pos, tables, table_width, heads, dim, rank,
                        cache_dim, page_size, num_pages);

@@ -1,0 +1,74 @@
+// Differential attention, the step behind the attention kernels.  Every head runs two softmax
+// maps over the same values (two heads of queries and keys to the attention kernels: map 0 of
+// head h is their head h, map 1 their head `heads + h`); here the second map is taken off the
+// first, the head's difference is divided by its root mean square (no weight), scaled by a
+// constant and, where the layer has one, multiplied element by element with the sigmoid of a
+// gate that was projected from the layer's input:
+//
+//   o = a0 - lambda a1,   out = o / sqrt(mean(o^2) + eps) * factor * sigmoid(g)
+//
+// over the head's `value_dim` values.  The difference, the norm and the sigmoid are 32-bit.
+// A wave per (token, head); a lane owns the values lane, lane + 64, ... (value_dim <= 256).
+#include <math.h>
+
+#include "common.h"
+#include "pagedserve_hip.h"
+
+template <typename T>
+__global__ __launch_bounds__(256) void differential_combine_kernel(
+    const T* __restrict__ ctx, int64_t ctx_ld, const float* __restrict__ lambda, float factor,
+    float eps, const float* __restrict__ gate, int64_t gate_ld, T* __restrict__ out, int64_t out_ld,
+    int tokens, int heads, int value_dim, int cache_dim) {
+  const int lane = threadIdx.x & 63;
+  const int64_t pair = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (pair >= (int64_t)tokens * heads) return;
+  const int64_t t = pair / heads;
+  const int head = (int)(pair - t * heads);
+  const T* first = ctx + t * ctx_ld + (int64_t)head * cache_dim;
+  const T* second = ctx + t * ctx_ld + (int64_t)(heads + head) * cache_dim;
+  const float l = lambda[0];
+  float o[4];
+  float squares = 0.f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int d = lane + 64 * i;
+    o[i] = d < value_dim ? to_float<T>(first[d]) - l * to_float<T>(second[d]) : 0.f;
+    squares = fmaf(o[i], o[i], squares);
+  }
+  const float scale = factor / sqrtf(wave_sum(squares) / (float)value_dim + eps);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int d = lane + 64 * i;
+    if (d >= value_dim) continue;
+    float v = o[i] * scale;
+    if (gate != nullptr) v *= 1.0f / (1.0f + expf(-gate[t * gate_ld + (int64_t)head * value_dim + d]));
+    out[t * out_ld + (int64_t)head * value_dim + d] = from_float<T>(v);
+  }
+}
+
+extern "C" int ps_differential_combine(const void* ctx, int64_t ctx_ld, const float* lambda,
+                                       float factor, float eps, const float* gate, int64_t gate_ld,
+                                       void* out, int64_t out_ld, int tokens, int heads,
+                                       int value_dim, int cache_dim, int dtype, void* stream) {
+  PS_REQUIRE(tokens >= 0 && heads > 0 && value_dim > 0 && value_dim <= 256 && cache_dim >= value_dim,
+             "ps_differential_combine: heads of %d values cached %d wide (1..256)", value_dim, cache_dim);
+  PS_REQUIRE(ctx_ld >= 2 * (int64_t)heads * cache_dim && out_ld >= (int64_t)heads * value_dim,
+             "ps_differential_combine: rows too short");
+  PS_REQUIRE(gate == nullptr || gate_ld >= (int64_t)heads * value_dim,
+             "ps_differential_combine: gate rows too short");
+  PS_REQUIRE(lambda != nullptr && eps > 0.f, "ps_differential_combine: lambda and a positive eps needed");
+  PS_REQUIRE(dtype == PS_F32 || dtype == PS_BF16, "ps_differential_combine: unknown dtype %d", dtype);
+  if (tokens == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  const dim3 grid((unsigned)(((int64_t)tokens * heads + 3) / 4));
+  if (dtype == PS_F32)
+    hipLaunchKernelGGL(differential_combine_kernel<float>, grid, dim3(256), 0, s, (const float*)ctx,
+                       ctx_ld, lambda, factor, eps, gate, gate_ld, (float*)out, out_ld, tokens, heads,
+                       value_dim, cache_dim);
+  else
+    hipLaunchKernelGGL(differential_combine_kernel<bf16_t>, grid, dim3(256), 0, s, (const bf16_t*)ctx,
+                       ctx_ld, lambda, factor, eps, gate, gate_ld, (bf16_t*)out, out_ld, tokens, heads,
+                       value_dim, cache_dim);
+  PS_CHECK_LAUNCH("ps_differential_combine");
+  return 0;
+}

@@ -6,6 +6,12 @@
 //   experts of the `keep` best groups may be chosen; the `top` largest s among them are, with
 //   the weights s * scale (not renormalised)
 //   out = sum over the chosen e of weight_e * W_down,e (silu(W_gate,e x) * (W_up,e x))
+//
+// Options of the router: sigmoid scores instead of the softmax; a correction per expert that is
+// added to the scores for the choice only (the weights use the scores without it; closed
+// experts count as minus infinity, since corrected scores may be negative); a group's score as
+// the sum of its `group_top` largest choice scores; weights divided by their sum (+ 1e-20).
+// Option of the experts: the plain form W_down,e relu(W_up,e x)^2 with one first matrix.
 #include <math.h>
 
 #include "common.h"
@@ -13,13 +19,45 @@
 
 #define MOE_MAX_EXPERTS 1024
 
+// What a router does beyond the softmax choice.
+struct RouteOptions {
+  int sigmoid;                 // scores are sigmoid(z) instead of softmax(z)
+  const float* correction;     // added to the scores for the choice (null: none)
+  int group_top;               // a group's score: the sum of this many largest choice scores
+  int normalise;               // the chosen weights are divided by their sum
+};
+
+// The sum of the `count` largest of choice[first .. first + size - 1] (count <= 8).
+__device__ inline float largest_sum(const float* choice, int first, int size, int count) {
+  int taken[8];
+  float total = 0.f;
+  if (count > size) count = size;
+  for (int r = 0; r < count; ++r) {
+    int best = -1;
+    float best_score = -INFINITY;
+    for (int e = first; e < first + size; ++e) {
+      bool used = false;
+      for (int q = 0; q < r; ++q) used = used || taken[q] == e;
+      if (!used && (best < 0 || choice[e] > best_score)) {
+        best_score = choice[e];
+        best = e;
+      }
+    }
+    taken[r] = best;
+    total += best_score;
+  }
+  return total;
+}
+
 // A block of one wave per token.  The logits are sums over the width dealt to the lanes; the
 // choice itself is a few dozen comparisons and is left to lane 0.
 template <typename T>
 __global__ __launch_bounds__(64) void moe_route_kernel(
     const T* __restrict__ x, int64_t x_ld, const float* __restrict__ w, int width, int experts,
-    int groups, int keep, int top, float scale, int* __restrict__ ids, float* __restrict__ weights) {
+    int groups, int keep, int top, float scale, RouteOptions options, int* __restrict__ ids,
+    float* __restrict__ weights) {
   __shared__ float s_score[MOE_MAX_EXPERTS];
+  __shared__ float s_choice[MOE_MAX_EXPERTS];
   __shared__ unsigned char s_open[MOE_MAX_EXPERTS];
   const int64_t t = blockIdx.x;
   const int lane = threadIdx.x;
@@ -33,16 +71,21 @@ __global__ __launch_bounds__(64) void moe_route_kernel(
   }
   __syncthreads();
   if (lane != 0) return;
-  float top_z = -INFINITY;
-  for (int e = 0; e < experts; ++e) top_z = fmaxf(top_z, s_score[e]);
-  float total = 0.f;
-  for (int e = 0; e < experts; ++e) {
-    s_score[e] = expf(s_score[e] - top_z);
-    total += s_score[e];
+  if (options.sigmoid) {
+    for (int e = 0; e < experts; ++e) s_score[e] = 1.0f / (1.0f + expf(-s_score[e]));
+  } else {
+    float top_z = -INFINITY;
+    for (int e = 0; e < experts; ++e) top_z = fmaxf(top_z, s_score[e]);
+    float total = 0.f;
+    for (int e = 0; e < experts; ++e) {
+      s_score[e] = expf(s_score[e] - top_z);
+      total += s_score[e];
+    }
+    const float inv = 1.0f / total;
+    for (int e = 0; e < experts; ++e) s_score[e] *= inv;
   }
-  const float inv = 1.0f / total;
   for (int e = 0; e < experts; ++e) {
-    s_score[e] *= inv;
+    s_choice[e] = s_score[e] + (options.correction ? options.correction[e] : 0.f);
     s_open[e] = groups <= 1 || keep >= groups;
   }
   if (groups > 1 && keep < groups) {
@@ -53,9 +96,8 @@ __global__ __launch_bounds__(64) void moe_route_kernel(
       float best_score = -INFINITY;
       for (int g = 0; g < groups; ++g) {
         if (s_open[g * size]) continue;
-        float score = -INFINITY;
-        for (int e = g * size; e < (g + 1) * size; ++e) score = fmaxf(score, s_score[e]);
-        if (score > best_score) {
+        const float score = largest_sum(s_choice, g * size, size, options.group_top);
+        if (best < 0 || score > best_score) {
           best_score = score;
           best = g;
         }
@@ -64,23 +106,25 @@ __global__ __launch_bounds__(64) void moe_route_kernel(
       for (int e = best * size; e < (best + 1) * size; ++e) s_open[e] = 1;
     }
   }
+  float chosen_sum = 0.f;
   for (int j = 0; j < top; ++j) {
     int best = -1;
     float best_score = -INFINITY;
     for (int e = 0; e < experts; ++e) {
-      if (s_open[e] == 1 && s_score[e] > best_score) {
-        best_score = s_score[e];
+      if (s_open[e] == 1 && (best < 0 || s_choice[e] > best_score)) {
+        best_score = s_choice[e];
         best = e;
       }
     }
-    if (best < 0) {       // (scores that are no numbers: any choice, but a valid one)
-      best = 0;
-      best_score = 0.f;
-    }
+    if (best < 0) best = 0;       // (scores that are no numbers: any choice, but a valid one)
     s_open[best] = 2;     // chosen: not again
     ids[t * top + j] = best;
-    weights[t * top + j] = best_score * scale;
+    const float own = s_score[best] == s_score[best] ? s_score[best] : 0.f;
+    weights[t * top + j] = own;
+    chosen_sum += own;
   }
+  const float factor = options.normalise ? scale / (chosen_sum + 1e-20f) : scale;
+  for (int j = 0; j < top; ++j) weights[t * top + j] *= factor;
 }
 
 // The same for up to 64 experts: a block of four waves per token, the waves share the experts'
@@ -89,7 +133,8 @@ __global__ __launch_bounds__(64) void moe_route_kernel(
 template <typename T>
 __global__ __launch_bounds__(256) void moe_route_wave_kernel(
     const T* __restrict__ x, int64_t x_ld, const float* __restrict__ w, int width, int experts,
-    int groups, int keep, int top, float scale, int* __restrict__ ids, float* __restrict__ weights) {
+    int groups, int keep, int top, float scale, RouteOptions options, int* __restrict__ ids,
+    float* __restrict__ weights) {
   __shared__ float s_score[64];
   __shared__ float s_group[64];
   const int64_t t = blockIdx.x;
@@ -107,18 +152,20 @@ __global__ __launch_bounds__(256) void moe_route_wave_kernel(
   const bool mine = lane < experts;
   const float z = mine ? s_score[lane] : -INFINITY;
   __syncthreads();
-  const float p = mine ? expf(z - wave_max(z)) : 0.f;
-  const float score = p / wave_sum(p);
+  float score;
+  if (options.sigmoid) {
+    score = mine ? 1.0f / (1.0f + expf(-z)) : 0.f;
+  } else {
+    const float p = mine ? expf(z - wave_max(z)) : 0.f;
+    score = p / wave_sum(p);
+  }
+  const float choice = score + ((mine && options.correction) ? options.correction[lane] : 0.f);
   bool open = mine;
   if (groups > 1 && keep < groups) {
     const int size = experts / groups;
-    s_score[lane] = score;
+    s_score[lane] = choice;
     __syncthreads();
-    if (lane < groups) {
-      float best = -INFINITY;
-      for (int e = lane * size; e < (lane + 1) * size; ++e) best = fmaxf(best, s_score[e]);
-      s_group[lane] = best;
-    }
+    if (lane < groups) s_group[lane] = largest_sum(s_score, lane * size, size, options.group_top);
     __syncthreads();
     if (mine) {
       const int g = lane / size;
@@ -131,26 +178,39 @@ __global__ __launch_bounds__(256) void moe_route_wave_kernel(
       open = ahead < keep;
     }
   }
+  int slot = -1;       // which of the token's choices this lane's expert is
   for (int j = 0; j < top; ++j) {
-    const float offer = open ? score : -1.f;
+    const float offer = open ? choice : -INFINITY;
     const float best = wave_max(offer);
-    const unsigned long long holders = __ballot(offer == best);
+    const unsigned long long holders = __ballot(open && offer == best);
     const int chosen = holders ? __builtin_ctzll(holders) : 0;
     if (lane == chosen) {
       open = false;
-      if (wave == 0) {
-        ids[t * top + j] = chosen;
-        weights[t * top + j] = (best < 0.f ? 0.f : best) * scale;
-      }
+      slot = j;
+      if (wave == 0) ids[t * top + j] = chosen;
     }
   }
+  const float own = (slot >= 0 && score == score) ? score : 0.f;
+  const float chosen_sum = wave_sum(own);
+  if (slot >= 0 && wave == 0) {
+    weights[t * top + slot] = options.normalise ? own / (chosen_sum + 1e-20f) * scale : own * scale;
+  }
+}
+
+// What a hidden column becomes: silu(g) * u of the gated form, relu(g)^2 of the plain one.
+template <bool GATED>
+__device__ inline float moe_activation(float g, float u) {
+  if (GATED) return g / (1.0f + expf(-g)) * u;
+  const float r = fmaxf(g, 0.f);
+  return r * r;
 }
 
 // hidden[(t, j), c] = silu(W_gate,e[c] . x_t) * (W_up,e[c] . x_t) for e = ids[t, j].  The
 // experts' first matrices lie one behind the other, [experts][gate rows | up rows][width].
 // A block of four waves per (token, choice) and 4 * ROWS hidden columns; the lanes share a dot
-// product's width.
-template <typename T, int ROWS>
+// product's width.  GATED false: the plain form, hidden = relu(W_up,e[c] . x_t)^2, the experts' first
+// matrices [experts][up rows][width].
+template <typename T, int ROWS, bool GATED>
 __global__ __launch_bounds__(256) void moe_hidden_kernel(
     const T* __restrict__ x, int64_t x_ld, const T* __restrict__ w1, const int* __restrict__ ids,
     T* __restrict__ hidden, int width, int inner) {
@@ -162,7 +222,7 @@ __global__ __launch_bounds__(256) void moe_hidden_kernel(
   for (int d = threadIdx.x; d < width; d += 256) s_x[d] = to_float<T>(x_row[d]);
   __syncthreads();
   const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
-  const T* base = w1 + (int64_t)e * 2 * inner * width;
+  const T* base = w1 + (int64_t)e * (GATED ? 2 : 1) * inner * width;
   const int first = (blockIdx.y * 4 + wave) * ROWS;
   for (int r = 0; r < ROWS; ++r) {
     const int c = first + r;
@@ -172,11 +232,11 @@ __global__ __launch_bounds__(256) void moe_hidden_kernel(
     float g = 0.f, u = 0.f;
     for (int d = lane; d < width; d += 64) {
       g = fmaf(to_float<T>(g_row[d]), s_x[d], g);
-      u = fmaf(to_float<T>(u_row[d]), s_x[d], u);
+      if (GATED) u = fmaf(to_float<T>(u_row[d]), s_x[d], u);
     }
     g = wave_sum(g);
-    u = wave_sum(u);
-    if (lane == 0) hidden[row_index * inner + c] = from_float<T>(g / (1.0f + expf(-g)) * u);
+    if (GATED) u = wave_sum(u);
+    if (lane == 0) hidden[row_index * inner + c] = from_float<T>(moe_activation<GATED>(g, u));
   }
 }
 
@@ -209,7 +269,8 @@ __global__ __launch_bounds__(256) void moe_down_kernel(
 }
 
 extern "C" int ps_moe_route(const void* x, int64_t x_ld, const float* w, int tokens, int width,
-                            int experts, int groups, int keep, int top, float scale, int* ids,
+                            int experts, int groups, int keep, int top, float scale, int sigmoid,
+                            const float* correction, int group_top, int normalise, int* ids,
                             float* weights, int dtype, void* stream) {
   PS_REQUIRE(tokens >= 0 && width > 0 && experts > 0 && experts <= MOE_MAX_EXPERTS,
              "ps_moe_route: %d experts, at most %d", experts, MOE_MAX_EXPERTS);
@@ -218,21 +279,24 @@ extern "C" int ps_moe_route(const void* x, int64_t x_ld, const float* w, int tok
   PS_REQUIRE(top >= 1 && top <= (experts / groups) * keep,
              "ps_moe_route: %d experts per token, %d may be chosen", top, (experts / groups) * keep);
   PS_REQUIRE(dtype == PS_F32 || dtype == PS_BF16, "ps_moe_route: unknown dtype %d", dtype);
+  PS_REQUIRE(group_top >= 1 && group_top <= 8,
+             "ps_moe_route: a group's score sums its %d largest scores, 1 to 8 are taken", group_top);
   if (tokens == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
+  const RouteOptions options = {sigmoid, correction, group_top, normalise};
   if (experts <= 64) {
     if (dtype == PS_F32)
       hipLaunchKernelGGL(moe_route_wave_kernel<float>, dim3(tokens), dim3(256), 0, s, (const float*)x,
-                         x_ld, w, width, experts, groups, keep, top, scale, ids, weights);
+                         x_ld, w, width, experts, groups, keep, top, scale, options, ids, weights);
     else
       hipLaunchKernelGGL(moe_route_wave_kernel<bf16_t>, dim3(tokens), dim3(256), 0, s, (const bf16_t*)x,
-                         x_ld, w, width, experts, groups, keep, top, scale, ids, weights);
+                         x_ld, w, width, experts, groups, keep, top, scale, options, ids, weights);
   } else if (dtype == PS_F32)
     hipLaunchKernelGGL(moe_route_kernel<float>, dim3(tokens), dim3(64), 0, s, (const float*)x, x_ld, w,
-                       width, experts, groups, keep, top, scale, ids, weights);
+                       width, experts, groups, keep, top, scale, options, ids, weights);
   else
     hipLaunchKernelGGL(moe_route_kernel<bf16_t>, dim3(tokens), dim3(64), 0, s, (const bf16_t*)x, x_ld,
-                       w, width, experts, groups, keep, top, scale, ids, weights);
+                       w, width, experts, groups, keep, top, scale, options, ids, weights);
   PS_CHECK_LAUNCH("ps_moe_route");
   return 0;
 }
@@ -262,7 +326,7 @@ __device__ inline void load8<float>(const float* p, float (&v)[8]) {
 
 // As moe_hidden_kernel for a width that is a multiple of 8: a wave owns ROWS hidden columns and
 // keeps the sums of their gate and up rows apart, so that 2 * ROWS loads are in flight per lane.
-template <typename T, int ROWS>
+template <typename T, int ROWS, bool GATED>
 __global__ __launch_bounds__(256) void moe_hidden_wide_kernel(
     const T* __restrict__ x, int64_t x_ld, const T* __restrict__ w1, const int* __restrict__ ids,
     T* __restrict__ hidden, int width, int inner) {
@@ -273,7 +337,7 @@ __global__ __launch_bounds__(256) void moe_hidden_wide_kernel(
   for (int d = threadIdx.x; d < width; d += 256) s_x[d] = to_float<T>(x_row[d]);
   __syncthreads();
   const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
-  const T* base = w1 + (int64_t)e * 2 * inner * width;
+  const T* base = w1 + (int64_t)e * (GATED ? 2 : 1) * inner * width;
   const int first = (blockIdx.y * 4 + wave) * ROWS;
   if (first >= inner) return;
   float g[ROWS], u[ROWS];
@@ -293,19 +357,19 @@ __global__ __launch_bounds__(256) void moe_hidden_wide_kernel(
     for (int r = 0; r < ROWS; ++r) {
       float a[8], b[8];
       load8<T>(rows_g[r] + d, a);
-      load8<T>(rows_g[r] + up + d, b);
+      if (GATED) load8<T>(rows_g[r] + up + d, b);
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
         g[r] = fmaf(a[i], xv[i], g[r]);
-        u[r] = fmaf(b[i], xv[i], u[r]);
+        if (GATED) u[r] = fmaf(b[i], xv[i], u[r]);
       }
     }
   }
 #pragma unroll
   for (int r = 0; r < ROWS; ++r) {
-    const float gs = wave_sum(g[r]), us = wave_sum(u[r]);
+    const float gs = wave_sum(g[r]), us = GATED ? wave_sum(u[r]) : 0.f;
     if (lane == 0 && first + r < inner)
-      hidden[row_index * inner + first + r] = from_float<T>(gs / (1.0f + expf(-gs)) * us);
+      hidden[row_index * inner + first + r] = from_float<T>(moe_activation<GATED>(gs, us));
   }
 }
 
@@ -398,10 +462,11 @@ typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 moe_bf16x8;
 // A tile of 128 sorted pairs times 128 weight rows of the tile's expert, k in stages of 32.
 // HIDDEN: the weight rows are 64 gate rows and the 64 up rows of the same hidden columns, and
 // hidden[pair, column] = silu(gate) * up; the rows of A are the pairs' tokens (pair / top).
-// Otherwise: 64 output columns (so that the narrower product still gives every compute unit a
+// MODE 2, the plain form's hidden rows: 64 up rows, hidden[pair, column] = relu(up)^2.
+// MODE 0: 64 output columns (so that the narrower product still gives every compute unit a
 // block), out[pair, column] = weights[pair] * sum; the rows of A are the pairs' hidden rows.
 // Four waves, 2 x 2: a wave has 64 pairs and 32 weight rows, twice in the first case.
-template <bool HIDDEN>
+template <int MODE>
 __global__ __launch_bounds__(256) void moe_grouped_kernel(
     const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __restrict__ w, int64_t expert_stride,
     int w_rows, int k, const int* __restrict__ order, const int* __restrict__ tile_expert, int top,
@@ -414,6 +479,8 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wave_m = wave >> 1, wave_n = wave & 1;
+  constexpr bool HIDDEN = MODE == 1;                     // gate and up rows side by side
+  constexpr bool FROM_TOKENS = MODE != 0;                // the rows of A are the pairs' tokens
   const int columns = HIDDEN ? w_rows / 2 : w_rows;      // output columns
   constexpr int NJ = HIDDEN ? 2 : 1;                     // runs of 64 weight rows in a stage
   const int n0 = blockIdx.y * 64;
@@ -430,7 +497,7 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
   for (int i = 0; i < 2; ++i) {
     const int a_pair = s_pair[a_row + i * 64];
     a_ok[i] = a_pair >= 0;
-    a_src[i] = a + (int64_t)(a_pair < 0 ? 0 : (HIDDEN ? a_pair / top : a_pair)) * lda + chunk;
+    a_src[i] = a + (int64_t)(a_pair < 0 ? 0 : (FROM_TOKENS ? a_pair / top : a_pair)) * lda + chunk;
     const int local = a_row + i * 64;      // 0..127
     int row;
     if (HIDDEN) row = (local < 64 ? 0 : columns) + n0 + (local & 63);
@@ -522,6 +589,9 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
       const int col = n0 + wave_n * 32 + (lane & 31);
       const float g = acc[r][0][i], u = acc[r][1][i];
       if (col < columns) hidden[(int64_t)pair * columns + col] = from_float<bf16_t>(g / (1.0f + expf(-g)) * u);
+    } else if (MODE == 2) {
+      const int col = n0 + wave_n * 32 + (lane & 31);
+      if (col < columns) hidden[(int64_t)pair * columns + col] = from_float<bf16_t>(moe_activation<false>(acc[r][0][i], 0.f));
     } else {
       const int col = n0 + wave_n * 32 + (lane & 31);
       if (col < columns) out[(int64_t)pair * out_ld + col] = weights[pair] * acc[r][0][i];
@@ -542,7 +612,8 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
 
 extern "C" int ps_moe_experts(const void* x, int64_t x_ld, const void* w1, const void* w2,
                               const int* ids, const float* weights, void* hidden, float* y,
-                              int tokens, int width, int inner, int top, int dtype, void* stream) {
+                              int tokens, int width, int inner, int top, int gated, int dtype,
+                              void* stream) {
   PS_REQUIRE(tokens >= 0 && width > 0 && inner > 0 && top > 0 && top <= 65535,
              "ps_moe_experts: bad sizes");
   PS_REQUIRE((size_t)width * 4 <= 64 * 1024 && (size_t)top * inner * 4 <= 64 * 1024,
@@ -554,16 +625,22 @@ extern "C" int ps_moe_experts(const void* x, int64_t x_ld, const void* w1, const
   // hidden columns / output columns per wave: four, or two while that still leaves the chip
   // short of blocks (a handful of decoded tokens)
   const bool few = (int64_t)tokens * ((width + 15) / 16) < 4 * ps_compute_units();
-#define PS_MOE_ROWS(T, ROWS)                                                                       \
+#define PS_MOE_HIDDEN(T, ROWS, GATED)                                                              \
   do {                                                                                             \
     const dim3 grid1(tokens, (inner + 4 * ROWS - 1) / (4 * ROWS), top);                            \
-    const dim3 grid2(tokens, (width + 4 * ROWS - 1) / (4 * ROWS));                                 \
     if (wide1)                                                                                     \
-      hipLaunchKernelGGL((moe_hidden_wide_kernel<T, ROWS>), grid1, dim3(256), (size_t)width * 4, s, \
-                         (const T*)x, x_ld, (const T*)w1, ids, (T*)hidden, width, inner);          \
+      hipLaunchKernelGGL((moe_hidden_wide_kernel<T, ROWS, GATED>), grid1, dim3(256),               \
+                         (size_t)width * 4, s, (const T*)x, x_ld, (const T*)w1, ids, (T*)hidden,   \
+                         width, inner);                                                            \
     else                                                                                           \
-      hipLaunchKernelGGL((moe_hidden_kernel<T, ROWS>), grid1, dim3(256), (size_t)width * 4, s,     \
-                         (const T*)x, x_ld, (const T*)w1, ids, (T*)hidden, width, inner);          \
+      hipLaunchKernelGGL((moe_hidden_kernel<T, ROWS, GATED>), grid1, dim3(256), (size_t)width * 4, \
+                         s, (const T*)x, x_ld, (const T*)w1, ids, (T*)hidden, width, inner);       \
+  } while (0)
+#define PS_MOE_ROWS(T, ROWS)                                                                       \
+  do {                                                                                             \
+    const dim3 grid2(tokens, (width + 4 * ROWS - 1) / (4 * ROWS));                                 \
+    if (gated) PS_MOE_HIDDEN(T, ROWS, true);                                                       \
+    else PS_MOE_HIDDEN(T, ROWS, false);                                                            \
     if (wide2)                                                                                     \
       hipLaunchKernelGGL((moe_down_wide_kernel<T, ROWS>), grid2, dim3(256), (size_t)top * inner * 4, \
                          s, (const T*)hidden, (const T*)w2, ids, weights, y, width, inner, top);   \
@@ -579,6 +656,7 @@ extern "C" int ps_moe_experts(const void* x, int64_t x_ld, const void* w1, const
     else PS_MOE_ROWS(bf16_t, 4);
   }
 #undef PS_MOE_ROWS
+#undef PS_MOE_HIDDEN
   PS_CHECK_LAUNCH("ps_moe_experts");
   return 0;
 }
@@ -591,7 +669,7 @@ extern "C" int ps_moe_experts_grouped(const void* x, int64_t x_ld, const void* w
                                       const int* ids, const float* weights, void* hidden,
                                       float* out, int* order, int* tile_expert, float* y,
                                       int tokens, int width, int inner, int experts, int top,
-                                      void* stream) {
+                                      int gated, void* stream) {
   PS_REQUIRE(tokens >= 0 && width > 0 && inner > 0 && top > 0 && experts > 0 &&
                  experts <= MOE_MAX_EXPERTS, "ps_moe_experts_grouped: bad sizes");
   PS_REQUIRE(width % 8 == 0 && inner % 8 == 0 && x_ld % 8 == 0,
@@ -602,11 +680,17 @@ extern "C" int ps_moe_experts_grouped(const void* x, int64_t x_ld, const void* w
   const int tiles = ps_moe_grouped_tiles(pairs, experts);
   hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(1024), 0, s, ids, pairs, experts, order, tile_expert,
                      tiles);
-  hipLaunchKernelGGL(moe_grouped_kernel<true>, dim3(tiles, (inner + 63) / 64), dim3(256), 0, s,
-                     (const bf16_t*)x, x_ld, (const bf16_t*)w1, (int64_t)2 * inner * width, 2 * inner,
-                     width, order, tile_expert, top, weights, (bf16_t*)hidden, (float*)nullptr,
-                     (int64_t)0);
-  hipLaunchKernelGGL(moe_grouped_kernel<false>, dim3(tiles, (width + 63) / 64), dim3(256), 0, s,
+  if (gated)
+    hipLaunchKernelGGL(moe_grouped_kernel<1>, dim3(tiles, (inner + 63) / 64), dim3(256), 0, s,
+                       (const bf16_t*)x, x_ld, (const bf16_t*)w1, (int64_t)2 * inner * width, 2 * inner,
+                       width, order, tile_expert, top, weights, (bf16_t*)hidden, (float*)nullptr,
+                       (int64_t)0);
+  else
+    hipLaunchKernelGGL(moe_grouped_kernel<2>, dim3(tiles, (inner + 63) / 64), dim3(256), 0, s,
+                       (const bf16_t*)x, x_ld, (const bf16_t*)w1, (int64_t)inner * width, inner,
+                       width, order, tile_expert, top, weights, (bf16_t*)hidden, (float*)nullptr,
+                       (int64_t)0);
+  hipLaunchKernelGGL(moe_grouped_kernel<0>, dim3(tiles, (width + 63) / 64), dim3(256), 0, s,
                      (const bf16_t*)hidden, (int64_t)inner, (const bf16_t*)w2, (int64_t)width * inner,
                      width, inner, order, tile_expert, top, weights, (bf16_t*)nullptr, out,
                      (int64_t)width);

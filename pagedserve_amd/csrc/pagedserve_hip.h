@@ -290,8 +290,8 @@ int ps_attention_prepare(const float* proj, int64_t ld, int q_col, int k_col, in
                          int rot_dims, void* v_first, const float* v_lambda, int v_mode,
                          const int* tok_item, const int* tok_pos, const int* tables,
                          int table_width, int tokens, int heads, int kv_heads, int key_dim,
-                         int value_dim, int cache_dim, int page_size, int num_pages, int dtype,
-                         void* stream);
+                         int value_dim, int cache_dim, int page_size, int num_pages, int v_heads,
+                         int store, int dtype, void* stream);
 // The same step for layers that treat every head on its own: the first rot_dims dimensions of
 // each query and key head rotated (halves != 0: dimension i with i + rot_dims / 2, else 2i with
 // 2i + 1; cosine and sine times magnitude), then, with head_norm, every head divided by its root
@@ -309,7 +309,8 @@ int ps_attention_prepare_heads(const float* proj, int64_t ld, int q_col, int k_c
 // cached row (k_pool: [pages, 1, page, cache_dim]) becomes [rms_norm(latent) * gamma | rotated key
 // part | zeros]; of every head's query row (cache_dim wide) the places rank .. rank + rot_dims - 1
 // get the rotated query part and the places behind zeros (the first `rank` are the caller's).
-int ps_latent_prepare(const float* proj, int64_t ld, int q_col, int kv_col, void* q_out,
+int ps_latent_prepare(const float* proj, int64_t ld, const float* queries, int64_t queries_ld,
+                      int q_col, int kv_col, void* q_out,
                       int64_t q_stride, void* k_pool, const float* gamma, float eps,
                       const float* freqs, int rot_dims, int halves, float magnitude,
                       const int* tok_item, const int* tok_pos, const int* tables, int table_width,
@@ -393,7 +394,7 @@ int ps_stream_step(float* h, const float* y, float factor, const float* column_s
                    int tokens, int width, int out_dtype, void* stream);
 // out[t, c] = silu(gu[t * ld + c]) * gu[t * ld + inner + c].
 int ps_silu_gate(const float* gu, int64_t ld, void* out, int64_t out_ld, int tokens, int inner,
-                 int dtype, void* stream);
+                 int activation, int dtype, void* stream);
 // p[t * ld + first + c] = silu(...) in place for c < count.
 int ps_silu_columns(float* p, int64_t ld, int first, int count, int tokens, void* stream);
 // y += share * (rms_norm(a) * wa + rms_norm(b) * wb) over rows of width floats; a and b are cleared.
@@ -427,13 +428,13 @@ int ps_lru_scan(const float* proj, int64_t ld, int y_col, int x_col, const float
 // (softmax over all experts of the 32-bit logits w x; only experts of the keep best of groups
 // equal groups of neighbours, a group's score being its largest s).
 int ps_moe_route(const void* x, int64_t x_ld, const float* w, int tokens, int width, int experts,
-                 int groups, int keep, int top, float scale, int* ids, float* weights, int dtype,
-                 void* stream);
+                 int groups, int keep, int top, float scale, int sigmoid, const float* correction,
+                 int group_top, int normalise, int* ids, float* weights, int dtype, void* stream);
 // y[t] += sum_j weights[t, j] W2[e] (silu(W1[e][:inner] x_t) * (W1[e][inner:] x_t)), e = ids[t, j];
 // w1: [experts, 2 * inner, width], w2: [experts, width, inner]; hidden: [tokens * top, inner] scratch.
 int ps_moe_experts(const void* x, int64_t x_ld, const void* w1, const void* w2, const int* ids,
                    const float* weights, void* hidden, float* y, int tokens, int width, int inner,
-                   int top, int dtype, void* stream);
+                   int top, int gated, int dtype, void* stream);
 // The same for many rows in bfloat16 (width and inner multiples of 8): the (token, choice) pairs
 // are sorted by expert into tiles of 128 and multiplied on the matrix cores.  order:
 // [tiles * 128] int and tile_expert: [tiles] int scratch with tiles = ps_moe_grouped_tiles(tokens *
@@ -442,7 +443,16 @@ int ps_moe_grouped_tiles(int pairs, int experts);
 int ps_moe_experts_grouped(const void* x, int64_t x_ld, const void* w1, const void* w2, const int* ids,
                            const float* weights, void* hidden, float* out, int* order,
                            int* tile_expert, float* y, int tokens, int width, int inner, int experts,
-                           int top, void* stream);
+                           int top, int gated, void* stream);
+
+// Differential attention behind the attention kernels: ctx holds two softmax maps per head over
+// the same values, map 0 of head h at head h and map 1 at head `heads + h`, cache_dim wide.
+// out[t, h, d] = (o / sqrt(mean_d(o^2) + eps)) * factor * sigmoid(gate[t, h * value_dim + d]) with
+// o = map0 - lambda[0] * map1 over the head's value_dim values (gate null: no gate).
+int ps_differential_combine(const void* ctx, int64_t ctx_ld, const float* lambda, float factor,
+                            float eps, const float* gate, int64_t gate_ld, void* out,
+                            int64_t out_ld, int tokens, int heads, int value_dim, int cache_dim,
+                            int dtype, void* stream);
 
 #ifdef __cplusplus
 }

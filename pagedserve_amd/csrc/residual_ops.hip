@@ -32,8 +32,8 @@ __global__ __launch_bounds__(256) void stream_step_kernel(
     normed[t * width + d] = from_float<T>(row[d] * inv * gamma[d]);
 }
 
-// out[t, c] = silu(gu[t, c]) * gu[t, inner + c]
-template <typename T>
+// out[t, c] = act(gu[t, c]) * gu[t, inner + c]; act: silu, or (GELU) the tanh form of gelu
+template <typename T, bool GELU>
 __global__ __launch_bounds__(256) void silu_gate_kernel(const float* __restrict__ gu, int64_t ld,
                                                         T* __restrict__ out, int64_t out_ld,
                                                         int inner) {
@@ -42,7 +42,7 @@ __global__ __launch_bounds__(256) void silu_gate_kernel(const float* __restrict_
   if (c >= inner) return;
   const float g = gu[t * ld + c];
   const float u = gu[t * ld + inner + c];
-  out[t * out_ld + c] = from_float<T>(g / (1.0f + expf(-g)) * u);
+  out[t * out_ld + c] = from_float<T>((GELU ? gelu_tanh_f(g) : g / (1.0f + expf(-g))) * u);
 }
 
 // p[t, c] <- silu(p[t, c]) for columns first .. first + count - 1 of rows ld floats apart
@@ -99,17 +99,22 @@ extern "C" int ps_stream_step(float* h, const float* y, float factor, const floa
 }
 
 extern "C" int ps_silu_gate(const float* gu, int64_t ld, void* out, int64_t out_ld, int tokens,
-                            int inner, int dtype, void* stream) {
+                            int inner, int activation, int dtype, void* stream) {
   PS_REQUIRE(tokens >= 0 && inner > 0 && ld >= 2 * (int64_t)inner && out_ld >= inner,
              "ps_silu_gate: bad sizes");
   PS_REQUIRE(dtype == PS_F32 || dtype == PS_BF16, "ps_silu_gate: unknown dtype %d", dtype);
   if (tokens == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
   const dim3 grid(tokens, (inner + 255) / 256);
-  if (dtype == PS_F32)
-    hipLaunchKernelGGL(silu_gate_kernel<float>, grid, dim3(256), 0, s, gu, ld, (float*)out, out_ld, inner);
+  PS_REQUIRE(activation == 0 || activation == 1, "ps_silu_gate: activation %d (0: silu, 1: gelu_tanh)", activation);
+  if (dtype == PS_F32 && activation)
+    hipLaunchKernelGGL((silu_gate_kernel<float, true>), grid, dim3(256), 0, s, gu, ld, (float*)out, out_ld, inner);
+  else if (dtype == PS_F32)
+    hipLaunchKernelGGL((silu_gate_kernel<float, false>), grid, dim3(256), 0, s, gu, ld, (float*)out, out_ld, inner);
+  else if (activation)
+    hipLaunchKernelGGL((silu_gate_kernel<bf16_t, true>), grid, dim3(256), 0, s, gu, ld, (bf16_t*)out, out_ld, inner);
   else
-    hipLaunchKernelGGL(silu_gate_kernel<bf16_t>, grid, dim3(256), 0, s, gu, ld, (bf16_t*)out, out_ld, inner);
+    hipLaunchKernelGGL((silu_gate_kernel<bf16_t, false>), grid, dim3(256), 0, s, gu, ld, (bf16_t*)out, out_ld, inner);
   PS_CHECK_LAUNCH("ps_silu_gate");
   return 0;
 }

@@ -40,7 +40,9 @@ _SIGNATURES = {
     "ps_attention_prepare": [c_void_p, c_int64, c_int, c_int, c_int, c_void_p, c_int64, c_void_p,
                              c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_int, c_void_p,
                              c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
-                             c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+                             c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "ps_differential_combine": [c_void_p, c_int64, c_void_p, c_float, c_float, c_void_p, c_int64,
+                                c_void_p, c_int64, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "ps_head_gate": [c_void_p, c_int64, c_void_p, c_int64, c_int, c_int, c_int, c_int, c_void_p],
     "ps_gla_decay": [c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_float, c_void_p, c_int,
                      c_int, c_int, c_void_p],
@@ -58,7 +60,7 @@ _SIGNATURES = {
                                    c_void_p, c_void_p, c_int, c_int, c_float, c_int, c_float, c_void_p,
                                    c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
                                    c_int, c_int, c_int, c_void_p],
-    "ps_latent_prepare": [c_void_p, c_int64, c_int, c_int, c_void_p, c_int64, c_void_p, c_void_p,
+    "ps_latent_prepare": [c_void_p, c_int64, c_void_p, c_int64, c_int, c_int, c_void_p, c_int64, c_void_p, c_void_p,
                           c_float, c_void_p, c_int, c_int, c_float, c_void_p, c_void_p, c_void_p, c_int,
                           c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "ps_block_linear": [c_void_p, c_int, c_int64, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int,
@@ -74,16 +76,16 @@ _SIGNATURES = {
     "ps_stream_step": [c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_float, c_void_p,
                        c_void_p, c_int, c_int, c_int, c_void_p],
     "ps_silu_columns": [c_void_p, c_int64, c_int, c_int, c_int, c_void_p],
-    "ps_silu_gate": [c_void_p, c_int64, c_void_p, c_int64, c_int, c_int, c_int, c_void_p],
+    "ps_silu_gate": [c_void_p, c_int64, c_void_p, c_int64, c_int, c_int, c_int, c_int, c_void_p],
     "ps_pair_norm_mix": [c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_float, c_void_p, c_int,
                          c_int, c_void_p],
     "ps_moe_route": [c_void_p, c_int64, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float,
-                     c_void_p, c_void_p, c_int, c_void_p],
+                     c_int, c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p],
     "ps_moe_experts_grouped": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
-                               c_void_p],
+                               c_int, c_void_p],
     "ps_moe_experts": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
-                       c_int, c_int, c_int, c_int, c_int, c_void_p],
+                       c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "ps_gla_output": [c_void_p, c_void_p, c_float, c_void_p, c_int64, c_void_p, c_int64, c_int,
                       c_int, c_int, c_int, c_void_p],
     "ps_softcap": [c_void_p, c_int64, c_int, c_int, c_float, c_void_p],
@@ -1220,11 +1222,14 @@ def streams_collapse(x, rows, out, width, streams):
 
 def attention_prepare(proj, columns, q_out, k_pool, v_pool, tok_item, tok_pos, tables, heads,
                       key_dim, value_dim, q_gamma=None, k_gamma=None, eps=1e-6, freqs=None,
-                      rot_dims=0, v_first=None, v_lambda=None, v_mode=0):
+                      rot_dims=0, v_first=None, v_lambda=None, v_mode=0, value_heads=0, store=True):
     """Norm, rotation, value mixing and cache write of an attention layer's projection
     (``csrc/pagedserve_hip.h: ps_attention_prepare``).  ``proj``: float ``[tokens, ld]`` with
     the query, key and value columns at ``columns = (q, k, v)``; the pools' head size is the
-    width that every head is stored with."""
+    width that every head is stored with.  ``value_heads`` (0: as many as key heads): the
+    projection holds that many value heads and key/value head j caches value head ``j %
+    value_heads``.  ``store=False``: only the queries are prepared, nothing is cached (a layer
+    that reads another layer's keys and values; its projection has no key or value columns)."""
     _check(proj, "proj", torch.float32, 2)
     ld = _rows(proj, "proj")
     tokens = proj.shape[0]
@@ -1234,7 +1239,13 @@ def attention_prepare(proj, columns, q_out, k_pool, v_pool, tok_item, tok_pos, t
     if q_out.shape[0] < tokens or q_out.shape[1] != heads * cache_dim:
         raise KernelError("attention_prepare: q_out must hold heads x cached head size per row")
     q_col, k_col, v_col = columns
-    if max(q_col + heads * key_dim, k_col + kv_heads * key_dim, v_col + kv_heads * value_dim) > proj.shape[1]:
+    value_heads = int(value_heads) or kv_heads
+    if value_heads < 1 or kv_heads % value_heads or (v_mode and value_heads != kv_heads):
+        raise KernelError(f"attention_prepare: {value_heads} value heads under {kv_heads} key heads")
+    needed = q_col + heads * key_dim
+    if store:
+        needed = max(needed, k_col + kv_heads * key_dim, v_col + value_heads * value_dim)
+    if needed > proj.shape[1]:
         raise KernelError("attention_prepare: the projection's rows are too short for its columns")
     _check_step_index(tok_item, tok_pos, tables, tokens)
     if q_gamma is not None:
@@ -1253,7 +1264,35 @@ def attention_prepare(proj, columns, q_out, k_pool, v_pool, tok_item, tok_pos, t
           k_pool.data_ptr(), v_pool.data_ptr(), _ptr(q_gamma), _ptr(k_gamma), float(eps), _ptr(freqs),
           int(rot_dims), _ptr(v_first), _ptr(v_lambda), int(v_mode), tok_item.data_ptr(),
           tok_pos.data_ptr(), tables.data_ptr(), tables.shape[1], tokens, heads, kv_heads, key_dim,
-          value_dim, cache_dim, page_size, pages, dtype_code(q_out.dtype), _stream())
+          value_dim, cache_dim, page_size, pages, value_heads, 1 if store else 0,
+          dtype_code(q_out.dtype), _stream())
+
+
+def differential_combine(context, lam, factor, eps, gate, out, heads, value_dim, cache_dim):
+    """Behind the attention kernels of a differential layer (``csrc/differential.hip``):
+    ``context [tokens, 2 * heads * cache_dim]`` holds map 0 of head h at head h and map 1 at head
+    ``heads + h``; ``out[t, h] = rms_norm(map0 - lam * map1) * factor * sigmoid(gate[t, h])`` over
+    the head's ``value_dim`` values, ``lam`` a float tensor of one number, ``gate`` float columns
+    ``[tokens, heads * value_dim]`` of a wider tensor or None."""
+    _check(context, "context", ndim=2)
+    _check(out, "out", context.dtype, 2)
+    tokens = context.shape[0]
+    if context.shape[1] != 2 * heads * cache_dim or context.stride(1) != 1:
+        raise KernelError(f"differential_combine: context must be [tokens, 2 x {heads} x {cache_dim}]")
+    if out.shape[0] < tokens or out.shape[1] != heads * value_dim or out.stride(1) != 1:
+        raise KernelError(f"differential_combine: out must be [>= {tokens}, {heads} x {value_dim}]")
+    if not 0 < value_dim <= min(cache_dim, 256):
+        raise KernelError(f"differential_combine: {value_dim} values in heads cached {cache_dim} wide (up to 256)")
+    _float_vector(lam, "lam", 1)
+    gate_ld = 0
+    if gate is not None:
+        _check(gate, "gate", torch.float32, 2)
+        if gate.shape[0] < tokens or gate.shape[1] != heads * value_dim or gate.stride(1) != 1:
+            raise KernelError("differential_combine: gate must be float [>= tokens, heads * value_dim]")
+        gate_ld = gate.stride(0)
+    _call("ps_differential_combine", context.data_ptr(), _rows(context, "context"), lam.data_ptr(),
+          float(factor), float(eps), _ptr(gate), gate_ld, out.data_ptr(), _rows(out, "out"), tokens,
+          heads, value_dim, cache_dim, dtype_code(context.dtype), _stream())
 
 
 def attention_prepare_heads(proj, columns, q_out, k_pool, v_pool, tok_item, tok_pos, tables, heads,
@@ -1288,12 +1327,14 @@ def attention_prepare_heads(proj, columns, q_out, k_pool, v_pool, tok_item, tok_
 
 
 def latent_prepare(proj, q_col, kv_col, q_out, k_pool, gamma, eps, tok_item, tok_pos, tables, heads,
-                   dim, rank, freqs=None, rot_dims=0, halves=True, magnitude=1.0):
+                   dim, rank, freqs=None, rot_dims=0, halves=True, magnitude=1.0, queries=None):
     """Latent attention between projection and attention: the token's cached row becomes
     ``[rms_norm(latent) * gamma | rotated key part | zeros]`` and every head's query row gets its
     rotated part at ``rank .. rank + rot_dims - 1`` and zeros behind (the first ``rank`` places
     are left to the caller).  ``proj``: per head ``[dim | rot_dims]`` from ``q_col`` on, ``[rank |
-    rot_dims]`` from ``kv_col`` on.  ``k_pool [pages, 1, page, cache_dim]``."""
+    rot_dims]`` from ``kv_col`` on.  ``queries``: float rows of their own that hold the heads'
+    queries from ``q_col`` on (queries that came through a latent), else they lie in ``proj``.
+    ``k_pool [pages, 1, page, cache_dim]``."""
     _check(proj, "proj", torch.float32, 2)
     _check(q_out, "q_out", ndim=2)
     _check(k_pool, "k_pool", q_out.dtype, 4)
@@ -1302,7 +1343,13 @@ def latent_prepare(proj, q_col, kv_col, q_out, k_pool, gamma, eps, tok_item, tok
     if kv_heads != 1 or not k_pool.is_contiguous() or cache_dim < rank + rot_dims:
         raise KernelError(f"latent_prepare: the pool {tuple(k_pool.shape)} must hold one row of at "
                           f"least {rank + rot_dims} per token")
-    if max(q_col + heads * (dim + rot_dims), kv_col + rank + rot_dims) > proj.shape[1]:
+    if queries is None:
+        queries = proj
+    else:
+        _check(queries, "queries", torch.float32, 2)
+        if queries.shape[0] < tokens:
+            raise KernelError("latent_prepare: too few rows of queries")
+    if q_col + heads * (dim + rot_dims) > queries.shape[1] or kv_col + rank + rot_dims > proj.shape[1]:
         raise KernelError("latent_prepare: the projection's rows are too short for its columns")
     if q_out.shape[0] < tokens or q_out.shape[1] != heads * cache_dim:
         raise KernelError(f"latent_prepare: q_out must be [>= {tokens}, {heads} x {cache_dim}]")
@@ -1310,7 +1357,8 @@ def latent_prepare(proj, q_col, kv_col, q_out, k_pool, gamma, eps, tok_item, tok
     _check_step_index(tok_item, tok_pos, tables, tokens)
     if rot_dims:
         _float_vector(freqs, "freqs", rot_dims // 2)
-    _call("ps_latent_prepare", proj.data_ptr(), _rows(proj, "proj"), int(q_col), int(kv_col),
+    _call("ps_latent_prepare", proj.data_ptr(), _rows(proj, "proj"), queries.data_ptr(),
+          _rows(queries, "queries"), int(q_col), int(kv_col),
           q_out.data_ptr(), _rows(q_out, "q_out"), k_pool.data_ptr(), gamma.data_ptr(), float(eps),
           _ptr(freqs), int(rot_dims), 1 if halves else 0, float(magnitude), tok_item.data_ptr(),
           tok_pos.data_ptr(), tables.data_ptr(), tables.shape[1], tokens, heads, int(dim), int(rank),
@@ -1635,15 +1683,21 @@ def stream_step(h, tokens, width, add=None, bias=None, norm=None, zero=None):
           _ptr(normed), _ptr(zero), tokens, width, code, _stream())
 
 
-def silu_gate(gu, out):
-    """``out[t, c] = silu(gu[t, c]) * gu[t, inner + c]`` for float ``gu`` of ``2 * inner`` columns."""
+GATE_ACTIVATIONS = {"silu": 0, "gelu_tanh": 1}
+
+
+def silu_gate(gu, out, activation="silu"):
+    """``out[t, c] = act(gu[t, c]) * gu[t, inner + c]`` for float ``gu`` of ``2 * inner`` columns;
+    ``act``: ``silu`` or ``gelu_tanh``."""
+    if activation not in GATE_ACTIVATIONS:
+        raise KernelError(f"silu_gate: activation {activation!r}; known: {', '.join(GATE_ACTIVATIONS)}")
     _check(gu, "gu", torch.float32, 2)
     _check(out, "out", ndim=2)
     tokens, inner = gu.shape[0], gu.shape[1] // 2
     if gu.shape[1] != 2 * inner or out.shape[0] < tokens or out.shape[1] != inner:
         raise KernelError("silu_gate: gu must hold twice out's columns")
     _call("ps_silu_gate", gu.data_ptr(), _rows(gu, "gu"), out.data_ptr(), _rows(out, "out"), tokens,
-          inner, dtype_code(out.dtype), _stream())
+          inner, GATE_ACTIVATIONS[activation], dtype_code(out.dtype), _stream())
 
 
 def silu_columns(rows, first, count):
@@ -1666,10 +1720,18 @@ def pair_norm_mix(a, b, weight_a, weight_b, eps, share, y, tokens, width):
           float(eps), float(share), y.data_ptr(), tokens, width, _stream())
 
 
-def moe_route(x, router, groups, keep, top, scale, ids, weights):
+def moe_route(x, router, groups, keep, top, scale, ids, weights, sigmoid=False, correction=None,
+              group_top=1, normalise=False):
     """The experts that every row of ``x`` chooses (``ids``, int32 ``[tokens, top]``) and their
-    weights (float): softmax over all experts of the 32-bit logits, group-limited choice, the
-    scores times ``scale`` (``csrc/moe.hip``)."""
+    weights (float): softmax (or ``sigmoid``) over all experts of the 32-bit logits, group-limited
+    choice, the scores times ``scale`` (``csrc/moe.hip``).  ``correction``: a float per expert
+    that is added to the scores for the choice only; ``group_top``: a group's score is the sum of
+    that many of its largest choice scores; ``normalise``: the chosen scores are divided by
+    their sum before ``scale``."""
+    if correction is not None:
+        _float_vector(correction, "correction", router.shape[0])
+    if not 1 <= int(group_top) <= 8:
+        raise KernelError(f"moe_route: group_top {group_top} must lie in 1..8")
     _check(x, "x", ndim=2)
     _check(router, "router", torch.float32, 2)
     tokens, width = x.shape
@@ -1682,7 +1744,8 @@ def moe_route(x, router, groups, keep, top, scale, ids, weights):
         if tensor.shape[0] < tokens or tensor.shape[1] != top or not tensor.is_contiguous():
             raise KernelError("moe_route: ids and weights must be contiguous [>= tokens, top]")
     _call("ps_moe_route", x.data_ptr(), x.stride(0), router.data_ptr(), tokens, width, experts,
-          int(groups), int(keep), int(top), float(scale), ids.data_ptr(), weights.data_ptr(),
+          int(groups), int(keep), int(top), float(scale), 1 if sigmoid else 0, _ptr(correction),
+          int(group_top), 1 if normalise else 0, ids.data_ptr(), weights.data_ptr(),
           dtype_code(x.dtype), _stream())
 
 
@@ -1699,7 +1762,7 @@ def moe_grouped_tiles(pairs, experts) -> int:
     return -(-pairs // MOE_TILE) + experts
 
 
-def moe_experts_grouped(x, w1, w2, ids, weights, hidden, out, order, tile_expert, y):
+def moe_experts_grouped(x, w1, w2, ids, weights, hidden, out, order, tile_expert, y, gated=True):
     """``moe_experts`` for many rows in bfloat16: the pairs sorted by expert, the products on the
     matrix cores.  ``out``: float ``[>= tokens * top, width]``, ``order``: int32 ``[>= tiles * MOE_TILE]``,
     ``tile_expert``: int32 ``[>= tiles]`` scratch with ``tiles = moe_grouped_tiles(tokens * top, experts)``."""
@@ -1708,9 +1771,9 @@ def moe_experts_grouped(x, w1, w2, ids, weights, hidden, out, order, tile_expert
     _check(w1, "w1", x.dtype, 3)
     _check(w2, "w2", x.dtype, 3)
     experts, inner = w2.shape[0], w2.shape[2]
-    if (tuple(w1.shape) != (experts, 2 * inner, width) or tuple(w2.shape) != (experts, width, inner)
+    if (tuple(w1.shape) != (experts, (2 if gated else 1) * inner, width) or tuple(w2.shape) != (experts, width, inner)
             or not (w1.is_contiguous() and w2.is_contiguous()) or x.stride(1) != 1):
-        raise KernelError("moe_experts_grouped: w1 [experts, 2 * inner, width] and w2 [experts, width, inner] needed")
+        raise KernelError("moe_experts_grouped: w1 [experts, (2) * inner, width] and w2 [experts, width, inner] needed")
     _check(ids, "ids", torch.int32, 2)
     _check(weights, "weights", torch.float32, 2)
     top = ids.shape[1]
@@ -1728,20 +1791,21 @@ def moe_experts_grouped(x, w1, w2, ids, weights, hidden, out, order, tile_expert
     _float_rows(y, "y", tokens, width)
     _call("ps_moe_experts_grouped", x.data_ptr(), x.stride(0), w1.data_ptr(), w2.data_ptr(), ids.data_ptr(),
           weights.data_ptr(), hidden.data_ptr(), out.data_ptr(), order.data_ptr(), tile_expert.data_ptr(),
-          y.data_ptr(), tokens, width, inner, experts, top, _stream())
+          y.data_ptr(), tokens, width, inner, experts, top, 1 if gated else 0, _stream())
 
 
-def moe_experts(x, w1, w2, ids, weights, hidden, y):
+def moe_experts(x, w1, w2, ids, weights, hidden, y, gated=True):
     """``y[t] += sum_j weights[t, j] W2[e] (silu(W1[e][:inner] x_t) * (W1[e][inner:] x_t))`` with
-    ``e = ids[t, j]``; ``w1``: ``[experts, 2 * inner, width]``, ``w2``: ``[experts, width, inner]``."""
+    ``e = ids[t, j]``; ``w1``: ``[experts, 2 * inner, width]``, ``w2``: ``[experts, width, inner]``.
+    ``gated=False``: the plain form ``W2[e] relu(W1[e] x_t)^2`` with ``w1 [experts, inner, width]``."""
     _check(x, "x", ndim=2)
     tokens, width = x.shape
     _check(w1, "w1", x.dtype, 3)
     _check(w2, "w2", x.dtype, 3)
     experts, inner = w2.shape[0], w2.shape[2]
-    if (tuple(w1.shape) != (experts, 2 * inner, width) or tuple(w2.shape) != (experts, width, inner)
+    if (tuple(w1.shape) != (experts, (2 if gated else 1) * inner, width) or tuple(w2.shape) != (experts, width, inner)
             or not (w1.is_contiguous() and w2.is_contiguous()) or x.stride(1) != 1):
-        raise KernelError("moe_experts: w1 [experts, 2 * inner, width] and w2 [experts, width, inner] needed")
+        raise KernelError("moe_experts: w1 [experts, (2) * inner, width] and w2 [experts, width, inner] needed")
     top = ids.shape[1]
     _check(ids, "ids", torch.int32, 2)
     _check(weights, "weights", torch.float32, 2)
@@ -1751,7 +1815,7 @@ def moe_experts(x, w1, w2, ids, weights, hidden, y):
     _float_rows(y, "y", tokens, width)
     _call("ps_moe_experts", x.data_ptr(), x.stride(0), w1.data_ptr(), w2.data_ptr(), ids.data_ptr(),
           weights.data_ptr(), hidden.data_ptr(), y.data_ptr(), tokens, width, inner, top,
-          dtype_code(x.dtype), _stream())
+          1 if gated else 0, dtype_code(x.dtype), _stream())
 
 
 def gla_output(o, weight, eps, gate, out, heads, value_dim):

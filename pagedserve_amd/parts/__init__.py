@@ -1,4 +1,5 @@
-from . import (attention, block, connection, embedding, feed_forward, latent_attention,  # noqa: F401
+from . import (attention, block, connection, differential_attention, embedding, feed_forward,  # noqa: F401
+               latent_attention,
                linear_attention, norm, position, side_by_side, state_space)  # noqa: F401  (register kinds)
 from .base import (CacheView, Embedding, FeedForward, Head, Mixer, Norm, PagedKVSpec, Part,
                    PositionEncoding, SlotStateSpec, StepContext, StepItem, Workspace)

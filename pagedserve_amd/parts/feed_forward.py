@@ -65,17 +65,22 @@ class DenseFeedForward(FeedForward):
 
 @register_feed_forward("gated")
 class GatedFeedForward(FeedForward):
-    """``residual += W_down (silu(W_gate x) * (W_up x))``, no biases.  One packed product gives
-    ``[gate | up]`` in float; the activation and the product of the halves are 32-bit."""
+    """``residual += W_down (act(W_gate x) * (W_up x))``, no biases; ``activation``: ``silu`` or
+    ``gelu_tanh``.  One packed product gives ``[gate | up]`` in float; the activation and the
+    product of the halves are 32-bit."""
 
     graph_safe = True
 
     accepts_pending_norm = True
 
-    def __init__(self, width: int, dtype, inner: int):
+    def __init__(self, width: int, dtype, inner: int, activation: str = "silu"):
+        if activation not in kernels.GATE_ACTIVATIONS:
+            raise ValueError(f"unknown gate activation {activation!r}; known: "
+                             f"{', '.join(kernels.GATE_ACTIVATIONS)}")
         self.width = width
         self.dtype = dtype
         self.inner = inner
+        self.activation = activation
         self._memo_up, self._memo_down = {}, {}
 
     def parameters(self):
@@ -98,7 +103,7 @@ class GatedFeedForward(FeedForward):
         kernels.linear(x, self.gate_up_weight, None, both, packed=self.gate_up_packed,
                        memo=site_memo(self._memo_up, ctx.workspace), shared=ctx.shared_calls)
         hidden = ctx.workspace.first_rows("ffn", self.inner, self.dtype, tokens)
-        kernels.silu_gate(both, hidden)
+        kernels.silu_gate(both, hidden, self.activation)
         kernels.linear(hidden, self.down_weight, None, residual, epilogue="residual",
                        packed=self.down_packed, memo=site_memo(self._memo_down, ctx.workspace),
                        shared=ctx.shared_calls)
@@ -106,7 +111,7 @@ class GatedFeedForward(FeedForward):
 
 @register_feed_forward("moe")
 class MixtureOfExperts(FeedForward):
-    """``experts`` small gated feed-forwards (no biases) of which each token uses ``top``:
+    """``experts`` small feed-forwards (no biases) of which each token uses ``top``:
 
         s = softmax(W_router x) over all experts, the logits in 32-bit
         experts form ``groups`` equal groups of neighbours; a group's score is its largest s and
@@ -115,20 +120,39 @@ class MixtureOfExperts(FeedForward):
 
     The weights are not renormalised.  The experts' matrices are stacked, ``[experts, gate rows
     | up rows, width]`` and ``[experts, width, inner]``; the choice stays on the device
-    (``csrc/moe.hip``)."""
+    (``csrc/moe.hip``).
+
+    Options: ``score="sigmoid"``: ``s = sigmoid(z)``; ``correction``: a number per expert
+    (``router.correction``) is added to ``s`` for the choice only, the weights use ``s`` without it;
+    ``group_top``: a group's score is the sum of that many of its largest choice scores;
+    ``normalise``: the chosen scores are divided by their sum (+ 1e-20) before ``scale``;
+    ``form="relu2"``: an expert is ``W_down,e relu(W_up,e x)^2`` (``up.weight [experts * inner,
+    width]``); ``shared_inner > 0``: one more expert of the same form and that inner width
+    (``shared.*``) runs for every token with weight one."""
 
     graph_safe = True
 
     accepts_pending_norm = False
 
+    SCORES = ("softmax", "sigmoid")
+    FORMS = ("gated_silu", "relu2")
+
     def __init__(self, width: int, dtype, inner: int, experts: int, top: int, groups: int = 1,
-                 keep: int = 1, scale: float = 1.0):
+                 keep: int = 1, scale: float = 1.0, score: str = "softmax", correction: bool = False,
+                 group_top: int = 1, normalise: bool = False, form: str = "gated_silu",
+                 shared_inner: int = 0):
         if groups < 1 or experts % groups:
             raise ValueError(f"{groups} groups do not divide {experts} experts")
         if not 1 <= keep <= groups:
             raise ValueError(f"keep ({keep}) must lie in 1..groups ({groups})")
         if not 1 <= top <= (experts // groups) * keep:
             raise ValueError(f"top ({top}) exceeds the experts that may be chosen")
+        if score not in self.SCORES:
+            raise ValueError(f"unknown router score {score!r}; known: {', '.join(self.SCORES)}")
+        if form not in self.FORMS:
+            raise ValueError(f"unknown expert form {form!r}; known: {', '.join(self.FORMS)}")
+        if not 1 <= group_top <= 8:
+            raise ValueError(f"group_top ({group_top}) must lie in 1..8")
         self.width = width
         self.dtype = dtype
         self.inner = inner
@@ -137,18 +161,42 @@ class MixtureOfExperts(FeedForward):
         self.groups = groups
         self.keep = keep
         self.scale = float(scale)
+        self.sigmoid = score == "sigmoid"
+        self.has_correction = bool(correction)
+        self.group_top = int(group_top)
+        self.normalise = bool(normalise)
+        self.gated = form == "gated_silu"
+        self.first_rows = (2 if self.gated else 1) * inner     # rows of an expert's first matrix
+        self.first_name = "gate_up.weight" if self.gated else "up.weight"
+        self.shared = None
+        if shared_inner:
+            if self.gated:
+                self.shared = GatedFeedForward(width, dtype, shared_inner)
+            else:
+                self.shared = DenseFeedForward(width, dtype, shared_inner, "relu2", bias=False)
 
     def parameters(self):
-        return {
+        params = {
             "router.weight": ParamSpec((self.experts, self.width), VECTOR),
-            "gate_up.weight": ParamSpec((self.experts * 2 * self.inner, self.width), MATRIX),
+            self.first_name: ParamSpec((self.experts * self.first_rows, self.width), MATRIX),
             "down.weight": ParamSpec((self.experts * self.width, self.inner), MATRIX),
         }
+        if self.has_correction:
+            params["router.correction"] = ParamSpec((self.experts,), VECTOR)
+        if self.shared is not None:
+            for name, spec in self.shared.parameters().items():
+                params["shared." + name] = spec
+        return params
 
     def bind(self, tensors):
         self.router_weight = tensors["router.weight"]
-        self.gate_up_weight = tensors["gate_up.weight"].view(self.experts, 2 * self.inner, self.width)
+        self.correction = tensors["router.correction"] if self.has_correction else None
+        self.first_weight = tensors[self.first_name].view(self.experts, self.first_rows, self.width)
+        if self.gated:
+            self.gate_up_weight = self.first_weight
         self.down_weight = tensors["down.weight"].view(self.experts, self.width, self.inner)
+        if self.shared is not None:
+            self.shared.bind({name: tensors["shared." + name] for name in self.shared.parameters()})
 
     def forward(self, x, residual, ctx):
         tokens = ctx.tokens
@@ -156,7 +204,8 @@ class MixtureOfExperts(FeedForward):
         ids = workspace.first_rows("moe_ids", self.top, torch.int32, tokens)
         weights = workspace.first_rows("moe_weights", self.top, torch.float32, tokens)
         kernels.moe_route(x, self.router_weight, self.groups, self.keep, self.top, self.scale, ids,
-                          weights)
+                          weights, sigmoid=self.sigmoid, correction=self.correction,
+                          group_top=self.group_top, normalise=self.normalise)
         most = workspace.max_rows * self.top
         hidden = workspace.rows("moe_hidden", self.inner, self.dtype, max_rows=most)
         if (tokens * self.top >= kernels.MOE_GROUPED_FROM
@@ -164,9 +213,12 @@ class MixtureOfExperts(FeedForward):
             # many rows: sorted by expert, tiles on the matrix cores
             tiles = kernels.moe_grouped_tiles(most, self.experts)
             kernels.moe_experts_grouped(
-                x, self.gate_up_weight, self.down_weight, ids, weights, hidden,
+                x, self.first_weight, self.down_weight, ids, weights, hidden,
                 workspace.rows("moe_out", self.width, torch.float32, max_rows=most),
                 workspace.flat("moe_order", tiles * kernels.MOE_TILE, torch.int32),
-                workspace.flat("moe_tiles", tiles, torch.int32), residual)
+                workspace.flat("moe_tiles", tiles, torch.int32), residual, gated=self.gated)
         else:
-            kernels.moe_experts(x, self.gate_up_weight, self.down_weight, ids, weights, hidden, residual)
+            kernels.moe_experts(x, self.first_weight, self.down_weight, ids, weights, hidden, residual,
+                                gated=self.gated)
+        if self.shared is not None:
+            self.shared.forward(x, residual, ctx)

@@ -33,12 +33,16 @@ class LatentAttention(Attention):
 
     Rotation: the ``rot_dim`` part whole, pairs laid out as halves by default, frequencies
     optionally stretched (``parts/position.py: rotary_frequencies``).  ``score_cap`` as in the
-    parent.  Norm, angles, scores, softmax and the gate's sigmoid are 32-bit."""
+    parent.  Norm, angles, scores, softmax and the gate's sigmoid are 32-bit.
+
+    ``query_rank > 0``: the queries come through a latent of their own, ``q = W_uq (rms_norm(W_dq
+    h) * gamma_q)`` (``query_down.weight``, ``query_norm.gamma``, ``query_up.weight``); the norm
+    runs inside the second product where that kernel takes it.  ``out_gate=False``: no gate."""
 
     def __init__(self, width: int, dtype, heads: int, dim: int, rot_dim: int, value_dim: int,
                  rank: int, scale: float, norm_eps: float = 1e-6, rotary_base: float = 10000.0,
                  rotary_scaling=None, rotary_layout: str = "halves", score_cap: float = 0.0,
-                 out_gate: bool = True):
+                 out_gate: bool = True, query_rank: int = 0):
         if rot_dim < 0 or rot_dim % 2:
             raise ValueError(f"rot_dim {rot_dim} must be even")
         cache_dim = -(-(rank + rot_dim) // 16) * 16
@@ -65,6 +69,9 @@ class LatentAttention(Attention):
         if self.score_cap < 0:
             raise ValueError("a score cap must be positive (0: none)")
         self.out_gate = bool(out_gate)
+        self.query_rank = int(query_rank)
+        if self.query_rank < 0:
+            raise ValueError("query_rank must not be negative (0: queries straight from the input)")
         # what the cache and the attention kernels see
         self.head_dim = cache_dim
         self.q_cols = heads * cache_dim
@@ -74,16 +81,26 @@ class LatentAttention(Attention):
         # the heads' value matrices and the gate lie between the attention and that projection)
         self.out_packed = None
         self._memo_in, self._memo_out, self._memo_attention = {}, {}, {}
+        self._memo_query_down, self._memo_query_up = {}, {}
 
     def _columns(self):
         """First column of the queries, of [latent | rotated key part] and of the gates in the
-        packed product, and its width."""
+        packed product, and its width.  Queries that come through a latent of their own are not
+        in that product."""
         q_col = 0
-        kv_col = q_col + self.heads * (self.dim + self.rot_dim)
+        kv_col = q_col + (0 if self.query_rank else self.heads * (self.dim + self.rot_dim))
         gate_col = kv_col + self.rank + self.rot_dim
         return q_col, kv_col, gate_col, gate_col + (self.heads * self.value_dim if self.out_gate else 0)
 
     def parameters(self):
+        params = self._own_parameters()
+        if self.query_rank:
+            params["query_down.weight"] = ParamSpec((self.query_rank, self.width), MATRIX)
+            params["query_norm.gamma"] = ParamSpec((self.query_rank,), VECTOR)
+            params["query_up.weight"] = ParamSpec((self.heads * (self.dim + self.rot_dim), self.query_rank), MATRIX)
+        return params
+
+    def _own_parameters(self):
         return {
             "in.weight": ParamSpec((self._columns()[3], self.width), MATRIX),
             "latent_norm.gamma": ParamSpec((self.rank,), VECTOR),
@@ -108,7 +125,14 @@ class LatentAttention(Attention):
             self.freqs = freqs.to(torch.float32).to(self.out_weight.device)
         self.in_packed = kernels.pack_decode_weight(self.in_weight)
         self.out_projection_packed = kernels.pack_decode_weight(self.out_weight)
-        for memo in (self._memo_in, self._memo_out, self._memo_attention):
+        if self.query_rank:
+            self.query_down_weight = tensors["query_down.weight"]
+            self.query_gamma = tensors["query_norm.gamma"]
+            self.query_up_weight = tensors["query_up.weight"]
+            self.query_down_packed = kernels.pack_decode_weight(self.query_down_weight)
+            self.query_up_packed = kernels.pack_decode_weight(self.query_up_weight)
+        for memo in (self._memo_in, self._memo_out, self._memo_attention, self._memo_query_down,
+                     self._memo_query_up):
             memo.clear()
 
     def cache_spec(self):
@@ -123,6 +147,21 @@ class LatentAttention(Attention):
         q_col, kv_col, gate_col, total = self._columns()
         proj, queries, _, gates = workspace.column_views(
             "latent_proj", total, torch.float32, tokens, (kv_col, gate_col - kv_col, total - gate_col))
+        if self.query_rank:
+            # the queries' own latent: its product in float, the norm inside the next product
+            # where the kernel takes it (x may be a norm that has not run: run it once for both)
+            if isinstance(x, kernels.PendingNorm):
+                x = x.materialize()
+            low = workspace.first_rows("latent_query_low", self.query_rank, torch.float32, tokens)
+            kernels.linear(x, self.query_down_weight, None, low, packed=self.query_down_packed,
+                           memo=site_memo(self._memo_query_down, workspace), shared=ctx.shared_calls)
+            normed = kernels.PendingNorm(low, self.query_gamma, None, self.norm_eps, True,
+                                         workspace.first_rows("latent_query_normed", self.query_rank,
+                                                              self.dtype, tokens))
+            queries = workspace.first_rows("latent_queries", self.heads * (self.dim + self.rot_dim),
+                                           torch.float32, tokens)
+            kernels.linear(normed, self.query_up_weight, None, queries, packed=self.query_up_packed,
+                           memo=site_memo(self._memo_query_up, workspace), shared=ctx.shared_calls)
         kernels.linear(x, self.in_weight, None, proj, packed=self.in_packed,
                        memo=site_memo(self._memo_in, workspace), shared=ctx.shared_calls)
         q = workspace.first_rows("latent_q", self.q_cols, self.dtype, tokens)
@@ -131,7 +170,8 @@ class LatentAttention(Attention):
         kernels.latent_prepare(proj, q_col, kv_col, q, cache.k_pool, self.latent_gamma, self.norm_eps,
                                ctx.tok_item, ctx.positions, tables, self.heads, self.dim, self.rank,
                                freqs=self.freqs, rot_dims=self.rot_dim, halves=self.rotary_halves,
-                               magnitude=self.rotary_magnitude)
+                               magnitude=self.rotary_magnitude,
+                               queries=queries if self.query_rank else None)
         self._gates = gates if self.out_gate else None
         context = workspace.first_rows("latent_context", self.q_cols, self.dtype, tokens)
         return self._attend(q, context, None, residual, ctx, cache, tables)
