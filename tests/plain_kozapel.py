@@ -274,3 +274,12 @@ def random_checkpoint(config, seed):
 
 def as_f64(tensors):
     return {name: value.to(F64) for name, value in tensors.items()}
+
+
+def greedy_generate(config, w, prompt, count):
+    """``count`` tokens after ``prompt``, each the most likely one (the whole sequence is run
+    again for every token: no cache to get wrong)."""
+    tokens = list(prompt)
+    for _ in range(count):
+        tokens.append(int(torch.argmax(forward(config, w, tokens)[-1])))
+    return tokens[len(prompt):]
