@@ -33,6 +33,7 @@ One JSON line is printed:
     python bench.py --design kosesun [--sizes small,small_narrow,medium]   Kosesun beside GPT-2 at equal size
     python bench.py --design zetunex [--sizes small,medium,small_many_experts]   Zetunex beside Kosesun at equal size
     python bench.py --design rezelix [--sizes small,medium,small_wide_heads]     Rezelix beside Zetunex at equal size
+    python bench.py --design kozapel [--sizes small,medium,small_narrow_maps]    Kozapel beside Kosesun at equal size
 
 ``--kernels`` times every kernel of a decode step (1, 8 and 64 requests over 1,024 keys), of
 the prefill step (2 x 1,024 tokens) and of a mixed step (32 decoded tokens beside a portion of
@@ -598,8 +599,50 @@ REZELIX_SIZES = {
     "small_wide_heads": (rezelix_shape(768, 12, 6, 2, 128, 3072, 50257, rank=96, rot_dim=32),
                          _dense_zetunex(768, 12, 6, 2, 128, 3072, 50257)),
 }
+def kozapel_shape(width, layers, heads, kv_heads, dim, vdim, ff, vocab, window=512, experts=8, top=2,
+                  rank=192, rot_dim=64, streams=4):
+    """A Kozapel configuration of a real model's layer sizes: of every four layers two are
+    differential attention under a window with keys and values of their own, the third is latent
+    attention (a latent of ``rank`` with a rotated part of ``rot_dim``, queries through a latent
+    half as wide as the model), the fourth differential attention on the second layer's keys and
+    values.  ``heads`` heads of two maps of ``dim`` each and values of ``vdim``.  Layers take turns
+    between a gated feed-forward and ``experts`` squared-ReLU experts of which ``top`` are chosen,
+    beside a shared one."""
+    listed = []
+    for index in range(layers):
+        kind = ("attention", "attention", "latent_attention", "attention")[index % 4]
+        if kind == "attention":
+            mixer = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": dim ** -0.5,
+                     "diff": 0.5, "mask": {"size": window}}
+            if index % 4 == 3:
+                mixer["kv_from"] = index - 2
+        else:
+            mixer = {"heads": heads, "dim": 2 * dim, "rot_dim": rot_dim, "vdim": 2 * dim, "kv_rank": rank,
+                     "q_rank": width // 2, "scale": (2 * dim + rot_dim) ** -0.5,
+                     "rot": {"dims": rot_dim, "base": 10000.0}}
+        entry = {"type": kind, "mixer": mixer}
+        if index % 2:
+            entry["mlp"] = {"kind": "moe", "expert": {"ff": ff // 2}, "shared": {"ff": ff // 2},
+                            "router": {"experts": experts, "top": top, "scale": 2.5,
+                                       "groups": {"count": 4, "keep": 2}}}
+        else:
+            entry["mlp"] = {"kind": "dense", "ff": ff}
+        listed.append(entry)
+    return {"architecture": "Kozapel", "vocab": vocab, "width": width, "streams": streams, "layers": listed,
+            "norm": {"eps": 1e-6}, "embedding": {"scale": width ** 0.5}}
+
+
+# name -> (Kozapel configuration, the Kosesun configuration of equal width, depth, inner width,
+# vocabulary and copies of the stream; a differential head's two maps count as two of its heads)
+KOZAPEL_SIZES = {
+    "small": (kozapel_shape(768, 12, 6, 2, 64, 128, 3072, 50257), kosesun_shape(768, 12, 12, 4, 64, 64, 3072, 50257)),
+    "medium": (kozapel_shape(1024, 24, 8, 2, 64, 128, 4096, 50257), kosesun_shape(1024, 24, 16, 4, 64, 64, 4096, 50257)),
+    # maps of 32 under values of 64, as many key/value heads as heads
+    "small_narrow_maps": (kozapel_shape(768, 12, 12, 12, 32, 64, 3072, 50257, rank=96, rot_dim=32),
+                          kosesun_shape(768, 12, 12, 12, 64, 64, 3072, 50257)),
+}
 DESIGNS = {"kosesun": (("kosesun", "gpt2"), DESIGN_SIZES), "zetunex": (("zetunex", "kosesun"), ZETUNEX_SIZES),
-           "rezelix": (("rezelix", "zetunex"), REZELIX_SIZES)}
+           "rezelix": (("rezelix", "zetunex"), REZELIX_SIZES), "kozapel": (("kozapel", "kosesun"), KOZAPEL_SIZES)}
 
 
 def design_comparison(args):
@@ -706,7 +749,7 @@ def main(argv=None):
     parser.add_argument("--rows", default="1,8,64", help="decode batch sizes of --kernels")
     parser.add_argument("--only", help="--kernels: only kernels whose name holds one of these (comma-separated)")
     parser.add_argument("--no-prefill", action="store_true", help="--kernels: decode tables only")
-    parser.add_argument("--design", choices=("kosesun", "zetunex", "rezelix"), default=None,
+    parser.add_argument("--design", choices=("kosesun", "zetunex", "rezelix", "kozapel"), default=None,
                         help="prefill and decode throughput of this design beside the closest other one at equal size")
     parser.add_argument("--sizes", default="small,small_narrow,medium", help="--design: which sizes")
     args = parser.parse_args(argv)

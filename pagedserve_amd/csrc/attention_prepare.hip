@@ -16,7 +16,10 @@
 //
 // `v_heads` < kv_heads: the projection holds that many value heads and key/value head j caches
 // value head j % v_heads (several maps of keys over the same values).  `store` 0: the layer reads
-// another layer's keys and values; only its queries are prepared.
+// another layer's keys and values; only its queries are prepared.  `q_maps` > 1: a query head has
+// `q_dim` dimensions of its own and query head j stands at places (j % q_maps) * q_dim onward of
+// its row, zeros elsewhere, so that it meets only its own run of a key head that holds q_maps
+// runs side by side (key_dim = q_maps * q_dim; no rotation then).
 #include <math.h>
 
 #include "common.h"
@@ -31,13 +34,13 @@ __global__ __launch_bounds__(1024) void attention_prepare_kernel(
     const float* __restrict__ v_lambda, int v_mode, const int* __restrict__ tok_item,
     const int* __restrict__ tok_pos, const int* __restrict__ tables, int table_width, int heads,
     int kv_heads, int key_dim, int value_dim, int cache_dim, int page_size, int num_pages,
-    int v_heads, int store) {
+    int v_heads, int store, int q_dim, int q_maps) {
   __shared__ float red[2][16];
   __shared__ float s_cos[128], s_sin[128];   // the token's angles, one per rotated pair of a head
   const int t = blockIdx.x;
   const float* row = proj + (int64_t)t * ld;
   const int pos = tok_pos[t];
-  const int q_cols = heads * key_dim, k_cols = kv_heads * key_dim;
+  const int q_cols = heads * q_dim, k_cols = kv_heads * key_dim;
   const int logical = pos / page_size;
   int page = -1;
   if (logical < table_width) page = tables[(int64_t)tok_item[t] * table_width + logical];
@@ -60,12 +63,17 @@ __global__ __launch_bounds__(1024) void attention_prepare_kernel(
     const int j = p.is_q ? i : i - q_pairs;
     p.head = j / half;
     p.d0 = (j - p.head * half) * 2;
-    const int src = (p.is_q ? q_col : k_col) + p.head * key_dim + p.d0;
+    // the head's own dimensions: `own` of them, from place `begin` of its row on
+    const int own = p.is_q ? q_dim : key_dim;
+    const int begin = p.is_q ? (p.head % q_maps) * q_dim : 0;
+    const int at = p.d0 - begin;
+    const int src = (p.is_q ? q_col : k_col) + p.head * own + at;
     const float* gamma = p.is_q ? q_gamma : k_gamma;
-    p.a = p.d0 < key_dim ? row[src] : 0.f;
-    p.b = p.d0 + 1 < key_dim ? row[src + 1] : 0.f;
-    p.wa = (gamma && p.d0 < key_dim) ? gamma[p.head * key_dim + p.d0] : 1.f;
-    p.wb = (gamma && p.d0 + 1 < key_dim) ? gamma[p.head * key_dim + p.d0 + 1] : 1.f;
+    const bool has_a = at >= 0 && at < own, has_b = at + 1 >= 0 && at + 1 < own;
+    p.a = has_a ? row[src] : 0.f;
+    p.b = has_b ? row[src + 1] : 0.f;
+    p.wa = (gamma && has_a) ? gamma[p.head * own + at] : 1.f;
+    p.wb = (gamma && has_b) ? gamma[p.head * own + at + 1] : 1.f;
     return p;
   };
   const int pairs = q_pairs + k_pairs;
@@ -148,7 +156,8 @@ extern "C" int ps_attention_prepare(const float* proj, int64_t ld, int q_col, in
                                     const int* tok_pos, const int* tables, int table_width,
                                     int tokens, int heads, int kv_heads, int key_dim,
                                     int value_dim, int cache_dim, int page_size, int num_pages,
-                                    int v_heads, int store, int dtype, void* stream) {
+                                    int v_heads, int store, int q_dim, int q_maps, int dtype,
+                                    void* stream) {
   PS_REQUIRE(tokens >= 0 && heads > 0 && kv_heads > 0 && key_dim > 0 && value_dim > 0 &&
                  page_size > 0 && num_pages > 0 && table_width > 0,
              "ps_attention_prepare: bad sizes");
@@ -166,6 +175,10 @@ extern "C" int ps_attention_prepare(const float* proj, int64_t ld, int q_col, in
   PS_REQUIRE(v_heads >= 1 && v_heads <= kv_heads && kv_heads % v_heads == 0 &&
                  (v_mode == 0 || v_heads == kv_heads),
              "ps_attention_prepare: %d value heads under %d key heads", v_heads, kv_heads);
+  PS_REQUIRE(q_maps >= 1 && q_dim >= 1 && q_maps * q_dim <= cache_dim &&
+                 (q_maps == 1 ? q_dim == key_dim : (rot_dims == 0 && q_maps * q_dim == key_dim)),
+             "ps_attention_prepare: %d runs of %d query dimensions do not fit keys of %d", q_maps, q_dim,
+             key_dim);
   PS_REQUIRE((q_gamma == nullptr && k_gamma == nullptr) || eps > 0.f, "ps_attention_prepare: eps must be positive");
   PS_REQUIRE(dtype == PS_F32 || dtype == PS_BF16, "ps_attention_prepare: unknown dtype %d", dtype);
   if (tokens == 0) return 0;
@@ -181,13 +194,13 @@ extern "C" int ps_attention_prepare(const float* proj, int64_t ld, int q_col, in
                        k_col, v_col, (float*)q_out, q_stride, (float*)k_pool, (float*)v_pool, q_gamma,
                        k_gamma, eps, freqs, rot_dims, (float*)v_first, v_lambda, v_mode, tok_item,
                        tok_pos, tables, table_width, heads, kv_heads, key_dim, value_dim, cache_dim,
-                       page_size, num_pages, v_heads, store);
+                       page_size, num_pages, v_heads, store, q_dim, q_maps);
   else
     hipLaunchKernelGGL(attention_prepare_kernel<bf16_t>, dim3(tokens), dim3(threads), 0, s, proj, ld, q_col,
                        k_col, v_col, (bf16_t*)q_out, q_stride, (bf16_t*)k_pool, (bf16_t*)v_pool,
                        q_gamma, k_gamma, eps, freqs, rot_dims, (bf16_t*)v_first, v_lambda, v_mode,
                        tok_item, tok_pos, tables, table_width, heads, kv_heads, key_dim, value_dim,
-                       cache_dim, page_size, num_pages, v_heads, store);
+                       cache_dim, page_size, num_pages, v_heads, store, q_dim, q_maps);
   PS_CHECK_LAUNCH("ps_attention_prepare");
   return 0;
 }

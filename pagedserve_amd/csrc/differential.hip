@@ -1,6 +1,6 @@
 // Differential attention, the step behind the attention kernels.  Every head runs two softmax
-// maps over the same values (two heads of queries and keys to the attention kernels: map 0 of
-// head h is their head h, map 1 their head `heads + h`); here the second map is taken off the
+// maps over the same values (two heads of queries to the attention kernels: map m of head h is
+// their head `m * heads + h`, or `2 * h + m`); here the second map is taken off the
 // first, the head's difference is divided by its root mean square (no weight), scaled by a
 // constant and, where the layer has one, multiplied element by element with the sigmoid of a
 // gate that was projected from the layer's input:
@@ -18,14 +18,14 @@ template <typename T>
 __global__ __launch_bounds__(256) void differential_combine_kernel(
     const T* __restrict__ ctx, int64_t ctx_ld, const float* __restrict__ lambda, float factor,
     float eps, const float* __restrict__ gate, int64_t gate_ld, T* __restrict__ out, int64_t out_ld,
-    int tokens, int heads, int value_dim, int cache_dim) {
+    int tokens, int heads, int value_dim, int cache_dim, int map_major) {
   const int lane = threadIdx.x & 63;
   const int64_t pair = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (pair >= (int64_t)tokens * heads) return;
   const int64_t t = pair / heads;
   const int head = (int)(pair - t * heads);
-  const T* first = ctx + t * ctx_ld + (int64_t)head * cache_dim;
-  const T* second = ctx + t * ctx_ld + (int64_t)(heads + head) * cache_dim;
+  const T* first = ctx + t * ctx_ld + (int64_t)(map_major ? head : 2 * head) * cache_dim;
+  const T* second = ctx + t * ctx_ld + (int64_t)(map_major ? heads + head : 2 * head + 1) * cache_dim;
   const float l = lambda[0];
   float o[4];
   float squares = 0.f;
@@ -49,7 +49,8 @@ __global__ __launch_bounds__(256) void differential_combine_kernel(
 extern "C" int ps_differential_combine(const void* ctx, int64_t ctx_ld, const float* lambda,
                                        float factor, float eps, const float* gate, int64_t gate_ld,
                                        void* out, int64_t out_ld, int tokens, int heads,
-                                       int value_dim, int cache_dim, int dtype, void* stream) {
+                                       int value_dim, int cache_dim, int map_major, int dtype,
+                                       void* stream) {
   PS_REQUIRE(tokens >= 0 && heads > 0 && value_dim > 0 && value_dim <= 256 && cache_dim >= value_dim,
              "ps_differential_combine: heads of %d values cached %d wide (1..256)", value_dim, cache_dim);
   PS_REQUIRE(ctx_ld >= 2 * (int64_t)heads * cache_dim && out_ld >= (int64_t)heads * value_dim,
@@ -64,11 +65,11 @@ extern "C" int ps_differential_combine(const void* ctx, int64_t ctx_ld, const fl
   if (dtype == PS_F32)
     hipLaunchKernelGGL(differential_combine_kernel<float>, grid, dim3(256), 0, s, (const float*)ctx,
                        ctx_ld, lambda, factor, eps, gate, gate_ld, (float*)out, out_ld, tokens, heads,
-                       value_dim, cache_dim);
+                       value_dim, cache_dim, map_major);
   else
     hipLaunchKernelGGL(differential_combine_kernel<bf16_t>, grid, dim3(256), 0, s, (const bf16_t*)ctx,
                        ctx_ld, lambda, factor, eps, gate, gate_ld, (bf16_t*)out, out_ld, tokens, heads,
-                       value_dim, cache_dim);
+                       value_dim, cache_dim, map_major);
   PS_CHECK_LAUNCH("ps_differential_combine");
   return 0;
 }

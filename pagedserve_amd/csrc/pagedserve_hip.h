@@ -291,7 +291,7 @@ int ps_attention_prepare(const float* proj, int64_t ld, int q_col, int k_col, in
                          const int* tok_item, const int* tok_pos, const int* tables,
                          int table_width, int tokens, int heads, int kv_heads, int key_dim,
                          int value_dim, int cache_dim, int page_size, int num_pages, int v_heads,
-                         int store, int dtype, void* stream);
+                         int store, int q_dim, int q_maps, int dtype, void* stream);
 // The same step for layers that treat every head on its own: the first rot_dims dimensions of
 // each query and key head rotated (halves != 0: dimension i with i + rot_dims / 2, else 2i with
 // 2i + 1; cosine and sine times magnitude), then, with head_norm, every head divided by its root
@@ -446,13 +446,14 @@ int ps_moe_experts_grouped(const void* x, int64_t x_ld, const void* w1, const vo
                            int top, int gated, void* stream);
 
 // Differential attention behind the attention kernels: ctx holds two softmax maps per head over
-// the same values, map 0 of head h at head h and map 1 at head `heads + h`, cache_dim wide.
+// the same values, cache_dim wide: map m of head h at head `m * heads + h` (map_major) or at head
+// `2 * h + m`.
 // out[t, h, d] = (o / sqrt(mean_d(o^2) + eps)) * factor * sigmoid(gate[t, h * value_dim + d]) with
 // o = map0 - lambda[0] * map1 over the head's value_dim values (gate null: no gate).
 int ps_differential_combine(const void* ctx, int64_t ctx_ld, const float* lambda, float factor,
                             float eps, const float* gate, int64_t gate_ld, void* out,
                             int64_t out_ld, int tokens, int heads, int value_dim, int cache_dim,
-                            int dtype, void* stream);
+                            int map_major, int dtype, void* stream);
 
 #ifdef __cplusplus
 }

@@ -40,9 +40,10 @@ _SIGNATURES = {
     "ps_attention_prepare": [c_void_p, c_int64, c_int, c_int, c_int, c_void_p, c_int64, c_void_p,
                              c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_int, c_void_p,
                              c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
-                             c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+                             c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+                             c_void_p],
     "ps_differential_combine": [c_void_p, c_int64, c_void_p, c_float, c_float, c_void_p, c_int64,
-                                c_void_p, c_int64, c_int, c_int, c_int, c_int, c_int, c_void_p],
+                                c_void_p, c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "ps_head_gate": [c_void_p, c_int64, c_void_p, c_int64, c_int, c_int, c_int, c_int, c_void_p],
     "ps_gla_decay": [c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_float, c_void_p, c_int,
                      c_int, c_int, c_void_p],
@@ -1222,14 +1223,18 @@ def streams_collapse(x, rows, out, width, streams):
 
 def attention_prepare(proj, columns, q_out, k_pool, v_pool, tok_item, tok_pos, tables, heads,
                       key_dim, value_dim, q_gamma=None, k_gamma=None, eps=1e-6, freqs=None,
-                      rot_dims=0, v_first=None, v_lambda=None, v_mode=0, value_heads=0, store=True):
+                      rot_dims=0, v_first=None, v_lambda=None, v_mode=0, value_heads=0, store=True,
+                      query_maps=1):
     """Norm, rotation, value mixing and cache write of an attention layer's projection
     (``csrc/pagedserve_hip.h: ps_attention_prepare``).  ``proj``: float ``[tokens, ld]`` with
     the query, key and value columns at ``columns = (q, k, v)``; the pools' head size is the
     width that every head is stored with.  ``value_heads`` (0: as many as key heads): the
     projection holds that many value heads and key/value head j caches value head ``j %
     value_heads``.  ``store=False``: only the queries are prepared, nothing is cached (a layer
-    that reads another layer's keys and values; its projection has no key or value columns)."""
+    that reads another layer's keys and values; its projection has no key or value columns).
+    ``query_maps > 1``: a key head holds that many runs of ``key_dim / query_maps`` dimensions side
+    by side, a query head has one run's dimensions, and query head j is written at the places of
+    run ``j % query_maps`` of its row, zeros elsewhere: it scores against its own run only."""
     _check(proj, "proj", torch.float32, 2)
     ld = _rows(proj, "proj")
     tokens = proj.shape[0]
@@ -1242,7 +1247,11 @@ def attention_prepare(proj, columns, q_out, k_pool, v_pool, tok_item, tok_pos, t
     value_heads = int(value_heads) or kv_heads
     if value_heads < 1 or kv_heads % value_heads or (v_mode and value_heads != kv_heads):
         raise KernelError(f"attention_prepare: {value_heads} value heads under {kv_heads} key heads")
-    needed = q_col + heads * key_dim
+    query_maps = int(query_maps)
+    if query_maps < 1 or key_dim % query_maps or (query_maps > 1 and (rot_dims or q_gamma is not None)):
+        raise KernelError(f"attention_prepare: {query_maps} runs in keys of {key_dim} (no rotation or norm with runs)")
+    q_dim = key_dim // query_maps
+    needed = q_col + heads * q_dim
     if store:
         needed = max(needed, k_col + kv_heads * key_dim, v_col + value_heads * value_dim)
     if needed > proj.shape[1]:
@@ -1264,14 +1273,14 @@ def attention_prepare(proj, columns, q_out, k_pool, v_pool, tok_item, tok_pos, t
           k_pool.data_ptr(), v_pool.data_ptr(), _ptr(q_gamma), _ptr(k_gamma), float(eps), _ptr(freqs),
           int(rot_dims), _ptr(v_first), _ptr(v_lambda), int(v_mode), tok_item.data_ptr(),
           tok_pos.data_ptr(), tables.data_ptr(), tables.shape[1], tokens, heads, kv_heads, key_dim,
-          value_dim, cache_dim, page_size, pages, value_heads, 1 if store else 0,
+          value_dim, cache_dim, page_size, pages, value_heads, 1 if store else 0, q_dim, query_maps,
           dtype_code(q_out.dtype), _stream())
 
 
-def differential_combine(context, lam, factor, eps, gate, out, heads, value_dim, cache_dim):
+def differential_combine(context, lam, factor, eps, gate, out, heads, value_dim, cache_dim, map_major=True):
     """Behind the attention kernels of a differential layer (``csrc/differential.hip``):
-    ``context [tokens, 2 * heads * cache_dim]`` holds map 0 of head h at head h and map 1 at head
-    ``heads + h``; ``out[t, h] = rms_norm(map0 - lam * map1) * factor * sigmoid(gate[t, h])`` over
+    ``context [tokens, 2 * heads * cache_dim]`` holds map m of head h at head ``m * heads + h``
+    (``map_major``) or ``2 * h + m``; ``out[t, h] = rms_norm(map0 - lam * map1) * factor * sigmoid(gate[t, h])`` over
     the head's ``value_dim`` values, ``lam`` a float tensor of one number, ``gate`` float columns
     ``[tokens, heads * value_dim]`` of a wider tensor or None."""
     _check(context, "context", ndim=2)
@@ -1292,7 +1301,7 @@ def differential_combine(context, lam, factor, eps, gate, out, heads, value_dim,
         gate_ld = gate.stride(0)
     _call("ps_differential_combine", context.data_ptr(), _rows(context, "context"), lam.data_ptr(),
           float(factor), float(eps), _ptr(gate), gate_ld, out.data_ptr(), _rows(out, "out"), tokens,
-          heads, value_dim, cache_dim, dtype_code(context.dtype), _stream())
+          heads, value_dim, cache_dim, 1 if map_major else 0, dtype_code(context.dtype), _stream())
 
 
 def attention_prepare_heads(proj, columns, q_out, k_pool, v_pool, tok_item, tok_pos, tables, heads,

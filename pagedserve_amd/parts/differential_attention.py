@@ -23,13 +23,18 @@ class DifferentialAttention(Attention):
         out = W_o (concat(o) * sigmoid(W_g h))                  (``out_gate``)
 
     No positions enter the scores.  ``window``: a query sees itself and the ``window - 1`` tokens
-    before it (0: all).  The attention kernels see ``2 H`` heads of ``dim`` over ``2 G``
-    key/value heads, map-major (map m of head j is their head ``m H + j``, of key head g their
-    ``m G + g``, so that grouped heads still find their key head by one division); the values of
-    key/value head g are cached under both of its maps.  Heads are cached ``max(dim, vdim)``
-    rounded up to 16 wide, zeros behind.  One launch behind the attention kernels takes the
-    difference, norms, scales and gates (``kernels.differential_combine``); scores, softmax, the
-    difference, the norm and the sigmoid are 32-bit.
+    before it (0: all).  The attention kernels see ``2 H`` query heads, one per map.  Where the two
+    maps' keys fit one cached head (``2 dim <= 256``) a key/value head is cached once: its two
+    maps' keys side by side, ``[k_0 | k_1]``, and its values, both ``max(2 dim, vdim)`` rounded
+    up to 16 wide; the query of map m stands at the places of ``k_m`` with zeros elsewhere, so its
+    product with the cached row is its own map's score, and the ``2 H / G`` query heads of a
+    key/value head read the same rows (head j's map m is the kernels' head ``2 j + m``).  Wider
+    maps are cached apart, ``2 G`` key/value heads of ``max(dim, vdim)``, map-major (map m of head
+    j is the kernels' head ``m H + j``, of key head g their ``m G + g``, so that grouped heads
+    still find their key head by one division), the values of head g under both of its maps.
+    One launch behind the attention kernels takes the difference, norms, scales and gates
+    (``kernels.differential_combine``); scores, softmax, the difference, the norm and the sigmoid
+    are 32-bit.
 
     ``reads_cache``: the layer has no key and value projections and reads the cache entry that
     another layer of the same geometry writes (``LayerCall.writes_cache = False``), with its own
@@ -52,11 +57,17 @@ class DifferentialAttention(Attention):
         self.true_heads = heads
         self.true_kv_heads = kv_heads
         # what the attention kernels see
-        self.heads = self.maps * heads
-        self.kv_heads = self.maps * kv_heads
-        self.key_dim = head_dim
+        self.map_dim = head_dim
         self.value_dim = value_dim
-        self.head_dim = -(-max(head_dim, value_dim) // 16) * 16
+        self.heads = self.maps * heads
+        self.packed = self.maps * head_dim <= 256
+        if self.packed:
+            self.kv_heads = kv_heads
+            self.key_dim = self.maps * head_dim
+        else:
+            self.kv_heads = self.maps * kv_heads
+            self.key_dim = head_dim
+        self.head_dim = -(-max(self.key_dim, value_dim) // 16) * 16
         self.scale = float(scale)
         self.diff = float(diff)
         self.window = int(window)
@@ -80,8 +91,8 @@ class DifferentialAttention(Attention):
     def _projection_columns(self):
         """First column of the queries, keys, values and gates in the packed product, and its width."""
         q_col = 0
-        k_col = q_col + self.heads * self.key_dim
-        v_col = k_col + (0 if self.reads_cache else self.kv_heads * self.key_dim)
+        k_col = q_col + self.heads * self.map_dim
+        v_col = k_col + (0 if self.reads_cache else self.maps * self.true_kv_heads * self.map_dim)
         gate_col = v_col + (0 if self.reads_cache else self.true_kv_heads * self.value_dim)
         return q_col, k_col, v_col, gate_col, gate_col + (self.true_heads * self.value_dim if self.out_gate else 0)
 
@@ -91,21 +102,23 @@ class DifferentialAttention(Attention):
             "out.weight": ParamSpec((self.width, self.true_heads * self.value_dim), MATRIX),
         }
         for name in ("lambda_q1", "lambda_k1", "lambda_q2", "lambda_k2"):
-            params[name] = ParamSpec((self.key_dim,), VECTOR)
+            params[name] = ParamSpec((self.map_dim,), VECTOR)
         return params
 
     def _map_major(self, rows, heads):
         """Rows laid out head by head as [map 0 | map 1] into all heads' map 0, then their map 1."""
-        return (rows.view(heads, self.maps, self.key_dim, -1).transpose(0, 1)
-                .reshape(heads * self.maps * self.key_dim, -1))
+        return (rows.view(heads, self.maps, self.map_dim, -1).transpose(0, 1)
+                .reshape(heads * self.maps * self.map_dim, -1))
 
     def bind(self, tensors):
         stored = tensors["qkv.weight"]
         q_col, k_col, v_col, _, _ = self._projection_columns()
-        weight = stored.clone()
-        weight[q_col:k_col] = self._map_major(stored[q_col:k_col], self.true_heads)
-        if not self.reads_cache:
-            weight[k_col:v_col] = self._map_major(stored[k_col:v_col], self.true_kv_heads)
+        weight = stored
+        if not self.packed:
+            weight = stored.clone()
+            weight[q_col:k_col] = self._map_major(stored[q_col:k_col], self.true_heads)
+            if not self.reads_cache:
+                weight[k_col:v_col] = self._map_major(stored[k_col:v_col], self.true_kv_heads)
         self.qkv_weight = weight
         self.out_weight = tensors["out.weight"]
         # one number for the layer, worked out once in 32-bit
@@ -135,7 +148,8 @@ class DifferentialAttention(Attention):
         q = workspace.first_rows("attn_q", self.q_cols, self.dtype, tokens)
         kernels.attention_prepare(proj, (q_col, k_col, v_col), q, cache.k_pool, cache.v_pool, ctx.tok_item,
                                   ctx.positions, tables, self.heads, self.key_dim, self.value_dim,
-                                  value_heads=self.true_kv_heads, store=not self.reads_cache)
+                                  value_heads=self.true_kv_heads, store=not self.reads_cache,
+                                  query_maps=self.maps if self.packed else 1)
         self._gates = gates if self.out_gate else None
         context = workspace.first_rows("attn", self.q_cols, self.dtype, tokens)
         return self._attend(q, context, None, residual, ctx, cache, tables)
@@ -143,7 +157,7 @@ class DifferentialAttention(Attention):
     def _project_out(self, context, residual, ctx):
         values = ctx.workspace.first_rows("diff_values", self.true_heads * self.value_dim, self.dtype, ctx.tokens)
         kernels.differential_combine(context, self.lam, 1.0 - self.diff, self.norm_eps, self._gates, values,
-                                     self.true_heads, self.value_dim, self.head_dim)
+                                     self.true_heads, self.value_dim, self.head_dim, map_major=not self.packed)
         kernels.linear(values, self.out_weight, None, residual, epilogue="residual",
                        packed=self.out_projection_packed, memo=site_memo(self._memo_out, ctx.workspace),
                        shared=ctx.shared_calls)

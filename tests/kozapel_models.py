@@ -82,8 +82,18 @@ MODEL_D = {
                _attention(2, 2, 128, 128, 0.05, 0.3, window=200, kv_from=1)],
 }
 
+# maps too wide to lie side by side in one cached head (two key/value heads per head's pair of
+# maps instead), two heads on one key/value head, a reader of such a layer, two copies of the stream
+MODEL_E = {
+    "architecture": "Kozapel", "vocab": 53, "width": 48, "streams": 2, "norm": {"eps": 1e-5},
+    "embedding": {"scale": 1.5},
+    "layers": [_attention(2, 1, 136, 40, 0.08, 0.4, window=10, mlp=_dense(64)),
+               _attention(2, 1, 136, 40, 0.07, 0.6, window=6, kv_from=0, mlp=_moe(8, 2, 1, 2, 2, 1.0, shared=8))],
+}
+
 # name -> (configuration, page size, seed)
-MODELS = {"A": (MODEL_A, 8, 0), "B": (MODEL_B, 16, 1), "C": (MODEL_C, 16, 2), "D": (MODEL_D, 4, 3)}
+MODELS = {"A": (MODEL_A, 8, 0), "B": (MODEL_B, 16, 1), "C": (MODEL_C, 16, 2), "D": (MODEL_D, 4, 3),
+          "E": (MODEL_E, 8, 4)}
 
 
 def write_folder(folder, raw, tensors):

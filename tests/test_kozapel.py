@@ -119,8 +119,8 @@ def test_every_stored_tensor_feeds_a_parameter_and_the_cache_is_what_the_layers_
     for group in groups:
         if group.values_in_keys:
             assert group.kv_heads == 1      # one latent row per token, read as keys and as values
-        else:
-            assert group.kv_heads % 2 == 0  # two maps of keys to a key/value head
+        elif raw["layers"][0]["mixer"].get("dim", 0) * 2 > 256:
+            assert group.kv_heads % 2 == 0  # maps too wide for one cached head: a head per map
     # experts stacked one behind the other, in their order
     for index, layer in enumerate(raw["layers"]):
         mlp = layer["mlp"]
@@ -132,12 +132,18 @@ def test_every_stored_tensor_feeds_a_parameter_and_the_cache_is_what_the_layers_
                                tensors[f"l{index}.mlp.e{mlp['router']['experts'] - 1}.down"])
             assert part.first_weight.shape[1] == ff
         if layer["type"] == "attention":
-            # the two maps of a head, stored side by side, lie map by map in the packed product
             part = model.blocks[index].mixer
             m = layer["mixer"]
             q = tensors[f"l{index}.mix.q"].view(m["heads"], 2, m["dim"], -1)
-            packed = part.qkv_weight[:2 * m["heads"] * m["dim"]].double().view(2, m["heads"], m["dim"], -1)
-            assert torch.equal(packed[1, m["heads"] - 1], q[m["heads"] - 1, 1])
+            rows = part.qkv_weight[:2 * m["heads"] * m["dim"]].double()
+            if part.packed:
+                # the two maps' keys lie side by side in one cached head, as they are stored
+                assert part.kv_heads == m["kv_heads"] and part.head_dim >= max(2 * m["dim"], m["vdim"])
+                assert torch.equal(rows.view(m["heads"], 2, m["dim"], -1), q)
+            else:
+                # a cached head per map: the maps of all heads lie map by map in the packed product
+                assert part.kv_heads == 2 * m["kv_heads"] and part.head_dim >= max(m["dim"], m["vdim"])
+                assert torch.equal(rows.view(2, m["heads"], m["dim"], -1)[1, m["heads"] - 1], q[m["heads"] - 1, 1])
             assert math.isclose(float(part.lam), plain.differential_lambda(tensors, f"l{index}.mix.", m["diff"]),
                                 rel_tol=1e-5)
 

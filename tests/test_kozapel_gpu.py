@@ -31,9 +31,10 @@ def _ints(values):
 
 # ---------------------------------------------------------------- kernels alone
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("map_major", [True, False])
 @pytest.mark.parametrize("heads,vdim,cache_dim,gated", [(4, 64, 64, True), (3, 20, 32, True), (2, 130, 144, False),
                                                         (1, 8, 16, True), (5, 256, 256, True)])
-def test_difference_of_the_maps_normed_scaled_and_gated(dtype, heads, vdim, cache_dim, gated):
+def test_difference_of_the_maps_normed_scaled_and_gated(dtype, heads, vdim, cache_dim, gated, map_major):
     kernels = _kernels()
     g = torch.Generator().manual_seed(heads * vdim)
     tokens = 11
@@ -43,8 +44,11 @@ def test_difference_of_the_maps_normed_scaled_and_gated(dtype, heads, vdim, cach
     out = torch.full((tokens, heads * vdim), 9.0, dtype=dtype, device="cuda")
     gate = gate_rows.cuda()[:, 3:3 + heads * vdim] if gated else None
     kernels.differential_combine(context.cuda(), torch.tensor([lam], device="cuda"), 1.0 - diff, eps, gate, out,
-                                 heads, vdim, cache_dim)
-    maps = context.double().view(tokens, 2, heads, cache_dim)[..., :vdim]
+                                 heads, vdim, cache_dim, map_major=map_major)
+    if map_major:
+        maps = context.double().view(tokens, 2, heads, cache_dim)[..., :vdim]
+    else:
+        maps = context.double().view(tokens, heads, 2, cache_dim)[..., :vdim].transpose(1, 2)
     expected = plain.rms_norm(maps[:, 0] - lam * maps[:, 1], None, eps) * (1.0 - diff)
     if gated:
         expected = expected * torch.sigmoid(gate_rows[:, 3:3 + heads * vdim].double().view(tokens, heads, vdim))
@@ -88,6 +92,7 @@ def test_two_maps_of_keys_stored_over_one_set_of_values(dtype, heads, kv_heads, 
     if not store:
         assert bool(torch.isnan(k_pool.float()).all()) and bool(torch.isnan(v_pool.float()).all())
         return
+    _two_maps_side_by_side(dtype, heads, kv_heads, dim, vdim, proj, q_col, k_col, v_col, tables, items, positions)
     keys = proj[:, k_col:k_col + seen_kv * dim].double().view(tokens, seen_kv, dim)
     values = proj[:, v_col:v_col + kv_heads * vdim].double().view(tokens, kv_heads, vdim)
     for t in range(tokens):
@@ -97,6 +102,35 @@ def test_two_maps_of_keys_stored_over_one_set_of_values(dtype, heads, kv_heads, 
             assert torch.allclose(row_k[:dim], keys[t, head], atol=tol, rtol=tol)
             assert torch.allclose(row_v[:vdim], values[t, head % kv_heads], atol=tol, rtol=tol)
             assert float(row_k[dim:].abs().sum()) == 0.0 and float(row_v[vdim:].abs().sum()) == 0.0
+
+
+def _two_maps_side_by_side(dtype, heads, kv_heads, dim, vdim, proj, q_col, k_col, v_col, tables, items, positions):
+    """The same projection cached the other way: a key/value head's two maps side by side in one
+    cached head, every query at the places of its own map and zeros elsewhere."""
+    kernels = _kernels()
+    tokens, page_size, pages = len(positions), 4, 9
+    cache_dim = -(-max(2 * dim, vdim) // 16) * 16
+    k_pool = torch.full((pages, kv_heads, page_size, cache_dim), float("nan"), dtype=dtype, device="cuda")
+    v_pool = torch.full_like(k_pool, float("nan"))
+    q_out = torch.full((tokens, 2 * heads * cache_dim), 5.0, dtype=dtype, device="cuda")
+    kernels.attention_prepare(proj.cuda(), (q_col, k_col, v_col), q_out, k_pool, v_pool, _ints(items),
+                              _ints(positions), tables.cuda(), 2 * heads, 2 * dim, vdim, query_maps=2)
+    tol = 1e-6 if dtype == torch.float32 else 1e-2
+    got_q = q_out.double().cpu().view(tokens, heads, 2, cache_dim)
+    want_q = proj[:, q_col:q_col + 2 * heads * dim].double().view(tokens, heads, 2, dim)
+    for m in range(2):
+        assert torch.allclose(got_q[:, :, m, m * dim:(m + 1) * dim], want_q[:, :, m], atol=tol, rtol=tol)
+        assert float(got_q[:, :, m, :m * dim].abs().sum()) == 0.0
+        assert float(got_q[:, :, m, (m + 1) * dim:].abs().sum()) == 0.0
+    keys = proj[:, k_col:k_col + 2 * kv_heads * dim].double().view(tokens, kv_heads, 2 * dim)
+    values = proj[:, v_col:v_col + kv_heads * vdim].double().view(tokens, kv_heads, vdim)
+    for t in range(tokens):
+        page, place = int(tables[items[t], positions[t] // page_size]), positions[t] % page_size
+        for head in range(kv_heads):
+            row_k, row_v = k_pool[page, head, place].double().cpu(), v_pool[page, head, place].double().cpu()
+            assert torch.allclose(row_k[:2 * dim], keys[t, head], atol=tol, rtol=tol)
+            assert torch.allclose(row_v[:vdim], values[t, head], atol=tol, rtol=tol)
+            assert float(row_k[2 * dim:].abs().sum()) == 0.0 and float(row_v[vdim:].abs().sum()) == 0.0
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
