@@ -462,7 +462,8 @@ typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 moe_bf16x8;
 // A tile of 128 sorted pairs times 128 weight rows of the tile's expert, k in stages of 32.
 // HIDDEN: the weight rows are 64 gate rows and the 64 up rows of the same hidden columns, and
 // hidden[pair, column] = silu(gate) * up; the rows of A are the pairs' tokens (pair / top).
-// MODE 2, the plain form's hidden rows: 64 up rows, hidden[pair, column] = relu(up)^2.
+// MODE 2, the plain form's hidden rows: 128 up rows, hidden[pair, column] = relu(up)^2 (a tile of
+// pairs is staged once for twice the columns).
 // MODE 0: 64 output columns (so that the narrower product still gives every compute unit a
 // block), out[pair, column] = weights[pair] * sum; the rows of A are the pairs' hidden rows.
 // Four waves, 2 x 2: a wave has 64 pairs and 32 weight rows, twice in the first case.
@@ -482,8 +483,8 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
   constexpr bool HIDDEN = MODE == 1;                     // gate and up rows side by side
   constexpr bool FROM_TOKENS = MODE != 0;                // the rows of A are the pairs' tokens
   const int columns = HIDDEN ? w_rows / 2 : w_rows;      // output columns
-  constexpr int NJ = HIDDEN ? 2 : 1;                     // runs of 64 weight rows in a stage
-  const int n0 = blockIdx.y * 64;
+  constexpr int NJ = MODE == 0 ? 1 : 2;                  // runs of 64 weight rows in a stage
+  const int n0 = blockIdx.y * (MODE == 2 ? 128 : 64);
   if (tid < MOE_TILE) s_pair[tid] = order[blockIdx.x * MOE_TILE + tid];
   __syncthreads();
   // staging: 16-byte chunks, 4 per row; A and W: 128 rows each, two chunks a thread
@@ -502,7 +503,7 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
     int row;
     if (HIDDEN) row = (local < 64 ? 0 : columns) + n0 + (local & 63);
     else row = n0 + local;
-    w_ok[i] = HIDDEN ? n0 + (local & 63) < columns : (local < 64 && row < w_rows);
+    w_ok[i] = HIDDEN ? n0 + (local & 63) < columns : ((MODE == 2 || local < 64) && row < w_rows);
     w_src[i] = w + (int64_t)e * expert_stride + (int64_t)(w_ok[i] ? row : 0) * k + chunk;
   }
   // a ring of MOE_DEPTH stages in registers keeps that many k tiles' loads in flight
@@ -590,8 +591,12 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
       const float g = acc[r][0][i], u = acc[r][1][i];
       if (col < columns) hidden[(int64_t)pair * columns + col] = from_float<bf16_t>(g / (1.0f + expf(-g)) * u);
     } else if (MODE == 2) {
-      const int col = n0 + wave_n * 32 + (lane & 31);
-      if (col < columns) hidden[(int64_t)pair * columns + col] = from_float<bf16_t>(moe_activation<false>(acc[r][0][i], 0.f));
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const int col = n0 + j * 64 + wave_n * 32 + (lane & 31);
+        if (col < columns)
+          hidden[(int64_t)pair * columns + col] = from_float<bf16_t>(moe_activation<false>(acc[r][j][i], 0.f));
+      }
     } else {
       const int col = n0 + wave_n * 32 + (lane & 31);
       if (col < columns) out[(int64_t)pair * out_ld + col] = weights[pair] * acc[r][0][i];
@@ -686,7 +691,7 @@ extern "C" int ps_moe_experts_grouped(const void* x, int64_t x_ld, const void* w
                        width, order, tile_expert, top, weights, (bf16_t*)hidden, (float*)nullptr,
                        (int64_t)0);
   else
-    hipLaunchKernelGGL(moe_grouped_kernel<2>, dim3(tiles, (inner + 63) / 64), dim3(256), 0, s,
+    hipLaunchKernelGGL(moe_grouped_kernel<2>, dim3(tiles, (inner + 127) / 128), dim3(256), 0, s,
                        (const bf16_t*)x, x_ld, (const bf16_t*)w1, (int64_t)inner * width, inner,
                        width, order, tile_expert, top, weights, (bf16_t*)hidden, (float*)nullptr,
                        (int64_t)0);
