@@ -278,7 +278,6 @@ extern "C" int ps_attention_decode_shared(const void* q, int64_t q_stride, const
   const int64_t need = (int64_t)count * heads * splits * (head_dim + 2);
   PS_REQUIRE(partial != nullptr && partial_floats >= need,
              "ps_attention_decode_shared: the records need %lld floats", (long long)need);
-  PS_REQUIRE(out != nullptr, "ps_attention_decode_shared: no output rows");
   if (count == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
   const bool same = v_pool == k_pool;
@@ -295,6 +294,7 @@ extern "C" int ps_attention_decode_shared(const void* q, int64_t q_stride, const
                      softcap * 1.4426950408889634f, ads_shift(page_size), ads_shift(head_dim / 8)};
   hipLaunchKernelGGL(attention_decode_shared_kernel, dim3(count, kv_heads * parts, splits), dim3(256), lds, s, a);
   PS_CHECK_LAUNCH("ps_attention_decode_shared");
+  if (out == nullptr) return 0;      // the records are all that is asked for: the caller merges them
   return ps_attention_reduce(partial, out, out_stride, tok_list, count, heads, head_dim, splits, gate, gate_ld,
                              PS_BF16, stream);
 }

@@ -27,24 +27,29 @@ struct RouteOptions {
   int normalise;               // the chosen weights are divided by their sum
 };
 
-// The sum of the `count` largest of choice[first .. first + size - 1] (count <= 8).
+// The sum of the `count` largest of choice[first .. first + size - 1].  The numbers are walked in
+// the order (larger first, lower index first); each round takes the first one behind the last
+// taken, so nothing has to be remembered but that one.
 __device__ inline float largest_sum(const float* choice, int first, int size, int count) {
-  int taken[8];
   float total = 0.f;
+  float last = INFINITY;
+  int last_at = -1;
   if (count > size) count = size;
   for (int r = 0; r < count; ++r) {
     int best = -1;
     float best_score = -INFINITY;
     for (int e = first; e < first + size; ++e) {
-      bool used = false;
-      for (int q = 0; q < r; ++q) used = used || taken[q] == e;
-      if (!used && (best < 0 || choice[e] > best_score)) {
-        best_score = choice[e];
+      const float v = choice[e];
+      const bool behind = v < last || (v == last && e > last_at);
+      if (behind && (best < 0 || v > best_score)) {
+        best_score = v;
         best = e;
       }
     }
-    taken[r] = best;
+    if (best < 0) break;      // (numbers that are no numbers)
     total += best_score;
+    last = best_score;
+    last_at = best;
   }
   return total;
 }

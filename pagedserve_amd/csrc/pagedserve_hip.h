@@ -454,6 +454,13 @@ int ps_differential_combine(const void* ctx, int64_t ctx_ld, const float* lambda
                             float eps, const float* gate, int64_t gate_ld, void* out,
                             int64_t out_ld, int tokens, int heads, int value_dim, int cache_dim,
                             int map_major, int dtype, void* stream);
+// The same for decoded tokens, from the records that ps_attention_decode_partial or
+// ps_attention_decode_shared (without output rows) left for 2 * heads heads of head_dim: the
+// ranges of both maps are merged in float, then as above.
+int ps_differential_merge(const float* partial, int64_t partial_floats, const int* tok_list, int count,
+                          const float* lambda, float factor, float eps, const float* gate,
+                          int64_t gate_ld, void* out, int64_t out_ld, int heads, int head_dim,
+                          int value_dim, int splits, int map_major, int dtype, void* stream);
 
 #ifdef __cplusplus
 }

@@ -44,6 +44,8 @@ _SIGNATURES = {
                              c_void_p],
     "ps_differential_combine": [c_void_p, c_int64, c_void_p, c_float, c_float, c_void_p, c_int64,
                                 c_void_p, c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "ps_differential_merge": [c_void_p, c_int64, c_void_p, c_int, c_void_p, c_float, c_float, c_void_p,
+                              c_int64, c_void_p, c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "ps_head_gate": [c_void_p, c_int64, c_void_p, c_int64, c_int, c_int, c_int, c_int, c_void_p],
     "ps_gla_decay": [c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_float, c_void_p, c_int,
                      c_int, c_int, c_void_p],
@@ -795,14 +797,17 @@ def attention_decode_shared(q, k_pool, v_pool, out, tok_item, tok_pos, tables, h
     to 16) and work on the matrix cores; ``v_pool`` may be ``k_pool``.  ``partial``: float scratch of
     ``count * heads * splits * (head_dim + 2)`` values, also with one range."""
     pages, kv_heads, page_size, head_dim, q_stride, out_stride, count = _attention_args(
-        q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, tok_list, direct_items=True)
+        q, k_pool, v_pool, q if out is None else out, tok_item, tok_pos, tables, heads, tok_list,
+        direct_items=True)
     if q.dtype != torch.bfloat16:
         raise KernelError("attention_decode_shared: bfloat16 only")
+    if out is None and gate is not None:
+        raise KernelError("attention_decode_shared: a gate needs output rows")
     _check(partial, "partial", torch.float32)
     if not partial.is_contiguous():
         raise KernelError("attention_decode_shared: scratch must be contiguous")
     _call("ps_attention_decode_shared", q.data_ptr(), q_stride, k_pool.data_ptr(), v_pool.data_ptr(),
-          out.data_ptr(), out_stride, partial.data_ptr(), partial.numel(), _ptr(tok_list), _ptr(tok_item),
+          _ptr(out), out_stride, partial.data_ptr(), partial.numel(), _ptr(tok_list), _ptr(tok_item),
           tok_pos.data_ptr(), tables.data_ptr(), tables.shape[1], count, heads, kv_heads, head_dim,
           page_size, pages, float(scale), int(window), int(splits), *_check_gate(gate, q.shape[0], heads),
           _check_cap(softcap), _stream())
@@ -1302,6 +1307,37 @@ def differential_combine(context, lam, factor, eps, gate, out, heads, value_dim,
     _call("ps_differential_combine", context.data_ptr(), _rows(context, "context"), lam.data_ptr(),
           float(factor), float(eps), _ptr(gate), gate_ld, out.data_ptr(), _rows(out, "out"), tokens,
           heads, value_dim, cache_dim, 1 if map_major else 0, dtype_code(context.dtype), _stream())
+
+
+def differential_merge(partial, count, splits, lam, factor, eps, gate, out, heads, value_dim, cache_dim,
+                       map_major=True, tok_list=None):
+    """``differential_combine`` for decoded tokens, from the records that ``attention_decode_partial``
+    or ``attention_decode_shared(out=None)`` left in ``partial`` for ``count`` tokens, ``2 * heads``
+    heads and ``splits`` key ranges: the ranges of both maps are merged in float, then the
+    difference, the norm, the factor and the gate; ``out [>= tokens, heads * value_dim]`` gets the
+    rows ``tok_list`` (None: the first ``count``)."""
+    _check(partial, "partial", torch.float32)
+    _check(out, "out", ndim=2)
+    if not partial.is_contiguous() or partial.numel() < count * 2 * heads * splits * (cache_dim + 2):
+        raise KernelError("differential_merge: too few records")
+    if out.shape[1] != heads * value_dim or out.stride(1) != 1 or (tok_list is None and out.shape[0] < count):
+        raise KernelError(f"differential_merge: out must be [>= {count}, {heads} x {value_dim}]")
+    if not 0 < value_dim <= min(cache_dim, 256) or not 1 <= splits <= 64:
+        raise KernelError(f"differential_merge: {value_dim} values in heads cached {cache_dim} wide, {splits} ranges")
+    _float_vector(lam, "lam", 1)
+    gate_ld = 0
+    if gate is not None:
+        _check(gate, "gate", torch.float32, 2)
+        if gate.shape[0] < out.shape[0] or gate.shape[1] != heads * value_dim or gate.stride(1) != 1:
+            raise KernelError("differential_merge: gate must be float [>= tokens, heads * value_dim]")
+        gate_ld = gate.stride(0)
+    if tok_list is not None:
+        _check(tok_list, "tok_list", torch.int32, 1)
+        if tok_list.numel() != count or not tok_list.is_contiguous():
+            raise KernelError("differential_merge: tok_list must name the tokens of the records")
+    _call("ps_differential_merge", partial.data_ptr(), partial.numel(), _ptr(tok_list), int(count),
+          lam.data_ptr(), float(factor), float(eps), _ptr(gate), gate_ld, out.data_ptr(), _rows(out, "out"),
+          heads, cache_dim, value_dim, int(splits), 1 if map_major else 0, dtype_code(out.dtype), _stream())
 
 
 def attention_prepare_heads(proj, columns, q_out, k_pool, v_pool, tok_item, tok_pos, tables, heads,

@@ -154,10 +154,40 @@ class DifferentialAttention(Attention):
         context = workspace.first_rows("attn", self.q_cols, self.dtype, tokens)
         return self._attend(q, context, None, residual, ctx, cache, tables)
 
+    def _attend(self, q, context, gates, residual, ctx, cache, tables):
+        """Steps of decoded tokens only: the split-KV kernels leave their records per key range and
+        one launch merges the ranges of both maps, takes the difference, norms and gates
+        (``kernels.differential_merge``).  Other steps take the parent's dispatch and the launch
+        that works on the attention's output rows."""
+        tokens = ctx.tokens
+        singles = ctx.single_tokens.numel() if ctx.single_tokens is not None else 0
+        if singles != tokens or not kernels.decode_supported(self.head_dim):
+            return super()._attend(q, context, gates, residual, ctx, cache, tables)
+        records = self._range_records(ctx)
+        if kernels.shared_decode_supported(self.dtype, self.heads, self.kv_heads, self.head_dim, None):
+            # many query heads (two maps of every head) to a key/value head: a tile of keys is
+            # loaded once for all of them
+            splits = self._shared_splits(singles, ctx.max_kv_len)
+            kernels.attention_decode_shared(q, cache.k_pool, cache.v_pool, None, None, ctx.positions, tables,
+                                            self.heads, self.scale, splits, records, window=self.window)
+        else:
+            splits, waves = self._splits(singles, ctx.max_kv_len)
+            kernels.attention_decode_partial(q, cache.k_pool, cache.v_pool, records, None, ctx.positions,
+                                             tables, self.heads, self.scale, splits, window=self.window,
+                                             waves=waves)
+        values = ctx.workspace.first_rows("diff_values", self.true_heads * self.value_dim, self.dtype, tokens)
+        kernels.differential_merge(records, tokens, splits, self.lam, 1.0 - self.diff, self.norm_eps,
+                                   self._gates, values, self.true_heads, self.value_dim, self.head_dim,
+                                   map_major=not self.packed)
+        self._project_values(values, residual, ctx)
+
     def _project_out(self, context, residual, ctx):
         values = ctx.workspace.first_rows("diff_values", self.true_heads * self.value_dim, self.dtype, ctx.tokens)
         kernels.differential_combine(context, self.lam, 1.0 - self.diff, self.norm_eps, self._gates, values,
                                      self.true_heads, self.value_dim, self.head_dim, map_major=not self.packed)
+        self._project_values(values, residual, ctx)
+
+    def _project_values(self, values, residual, ctx):
         kernels.linear(values, self.out_weight, None, residual, epilogue="residual",
                        packed=self.out_projection_packed, memo=site_memo(self._memo_out, ctx.workspace),
                        shared=ctx.shared_calls)

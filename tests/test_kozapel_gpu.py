@@ -57,6 +57,41 @@ def test_difference_of_the_maps_normed_scaled_and_gated(dtype, heads, vdim, cach
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("map_major", [True, False])
+@pytest.mark.parametrize("heads,vdim,cache_dim,splits", [(4, 64, 64, 5), (3, 20, 32, 1), (2, 130, 144, 64), (1, 8, 16, 9)])
+def test_ranges_of_both_maps_merged_and_combined_in_one_launch(dtype, heads, vdim, cache_dim, splits, map_major):
+    """Records per (token, head, key range) as the split-KV kernels leave them (accumulators, the
+    running maximum in units of log 2, the sum; a range that saw no key has minus infinity and
+    zeros), for a list of tokens of a larger step."""
+    kernels = _kernels()
+    g = torch.Generator().manual_seed(heads + splits)
+    rows, tok_list = 9, [7, 0, 3, 4]
+    count = len(tok_list)
+    acc = torch.randn((count, 2 * heads, splits, cache_dim), generator=g)
+    top = torch.randn((count, 2 * heads, splits), generator=g) * 3
+    total = torch.rand((count, 2 * heads, splits), generator=g) + 0.5
+    if splits > 1:
+        acc[:, :, 1], top[:, :, 1], total[:, :, 1] = 0.0, float("-inf"), 0.0
+    records = torch.cat([acc, top[..., None], total[..., None]], dim=-1).contiguous()
+    gate_rows = torch.randn((rows, heads * vdim + 5), generator=g)
+    lam, diff, eps = 0.61, 0.3, 1e-5
+    out = torch.full((rows, heads * vdim), 9.0, dtype=dtype, device="cuda")
+    kernels.differential_merge(records.cuda().reshape(-1), count, splits, torch.tensor([lam], device="cuda"),
+                               1.0 - diff, eps, gate_rows.cuda()[:, 2:2 + heads * vdim], out, heads, vdim,
+                               cache_dim, map_major=map_major, tok_list=_ints(tok_list))
+    weight = torch.exp2(top.double() - top.double().max(-1, keepdim=True).values)
+    merged = ((acc.double() * weight[..., None]).sum(2) / (total.double() * weight).sum(-1)[..., None])[..., :vdim]
+    maps = merged.view(count, 2, heads, vdim) if map_major else merged.view(count, heads, 2, vdim).transpose(1, 2)
+    expected = plain.rms_norm(maps[:, 0] - lam * maps[:, 1], None, eps) * (1.0 - diff)
+    expected = expected * torch.sigmoid(gate_rows[tok_list, 2:2 + heads * vdim].double().view(count, heads, vdim))
+    tol = 3e-5 if dtype == torch.float32 else 2e-2
+    got = out.double().cpu()
+    assert torch.allclose(got[tok_list].view(count, heads, vdim), expected, atol=tol, rtol=tol)
+    untouched = [row for row in range(rows) if row not in tok_list]
+    assert float((got[untouched] - 9.0).abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("heads,kv_heads,dim,vdim,store", [(4, 2, 16, 24, True), (3, 3, 12, 20, True),
                                                            (4, 1, 64, 32, True), (2, 1, 8, 8, False)])
 def test_two_maps_of_keys_stored_over_one_set_of_values(dtype, heads, kv_heads, dim, vdim, store):
