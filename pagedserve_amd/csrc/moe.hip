@@ -25,6 +25,9 @@ struct RouteOptions {
   const float* correction;     // added to the scores for the choice (null: none)
   int group_top;               // a group's score: the sum of this many largest choice scores
   int normalise;               // the chosen weights are divided by their sum
+  int fixed;                   // experts behind the routed ones that every token uses with weight 1:
+                               // a row of ids and weights is [top chosen | fixed], the fixed ones
+                               // numbered from `experts` on
 };
 
 // The sum of the `count` largest of choice[first .. first + size - 1].  The numbers are walked in
@@ -54,6 +57,26 @@ __device__ inline float largest_sum(const float* choice, int first, int size, in
   return total;
 }
 
+// A lane's share of the dot product of a token's row with an expert's router row: four strides
+// of the wave at a time, so that eight loads are on their way together instead of two.
+template <typename T>
+__device__ inline float router_dot(const T* __restrict__ row, const float* __restrict__ w_row, int width,
+                                   int lane) {
+  float sum = 0.f;
+  int d = lane;
+  for (; d + 192 < width; d += 256) {
+    const float x0 = to_float<T>(row[d]), x1 = to_float<T>(row[d + 64]);
+    const float x2 = to_float<T>(row[d + 128]), x3 = to_float<T>(row[d + 192]);
+    const float w0 = w_row[d], w1 = w_row[d + 64], w2 = w_row[d + 128], w3 = w_row[d + 192];
+    sum = fmaf(x0, w0, sum);
+    sum = fmaf(x1, w1, sum);
+    sum = fmaf(x2, w2, sum);
+    sum = fmaf(x3, w3, sum);
+  }
+  for (; d < width; d += 64) sum = fmaf(to_float<T>(row[d]), w_row[d], sum);
+  return sum;
+}
+
 // A block of one wave per token.  The logits are sums over the width dealt to the lanes; the
 // choice itself is a few dozen comparisons and is left to lane 0.
 template <typename T>
@@ -68,14 +91,12 @@ __global__ __launch_bounds__(64) void moe_route_kernel(
   const int lane = threadIdx.x;
   const T* row = x + t * x_ld;
   for (int e = 0; e < experts; ++e) {
-    const float* w_row = w + (int64_t)e * width;
-    float sum = 0.f;
-    for (int d = lane; d < width; d += 64) sum = fmaf(to_float<T>(row[d]), w_row[d], sum);
-    sum = wave_sum(sum);
+    const float sum = wave_sum(router_dot<T>(row, w + (int64_t)e * width, width, lane));
     if (lane == 0) s_score[e] = sum;
   }
   __syncthreads();
   if (lane != 0) return;
+  const int cols = top + options.fixed;
   if (options.sigmoid) {
     for (int e = 0; e < experts; ++e) s_score[e] = 1.0f / (1.0f + expf(-s_score[e]));
   } else {
@@ -123,13 +144,17 @@ __global__ __launch_bounds__(64) void moe_route_kernel(
     }
     if (best < 0) best = 0;       // (scores that are no numbers: any choice, but a valid one)
     s_open[best] = 2;     // chosen: not again
-    ids[t * top + j] = best;
+    ids[t * cols + j] = best;
     const float own = s_score[best] == s_score[best] ? s_score[best] : 0.f;
-    weights[t * top + j] = own;
+    weights[t * cols + j] = own;
     chosen_sum += own;
   }
   const float factor = options.normalise ? scale / (chosen_sum + 1e-20f) : scale;
-  for (int j = 0; j < top; ++j) weights[t * top + j] *= factor;
+  for (int j = 0; j < top; ++j) weights[t * cols + j] *= factor;
+  for (int j = 0; j < options.fixed; ++j) {
+    ids[t * cols + top + j] = experts + j;
+    weights[t * cols + top + j] = 1.0f;
+  }
 }
 
 // The same for up to 64 experts: a block of four waves per token, the waves share the experts'
@@ -146,10 +171,7 @@ __global__ __launch_bounds__(256) void moe_route_wave_kernel(
   const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
   const T* row = x + t * x_ld;
   for (int e = wave; e < experts; e += 4) {
-    const float* w_row = w + (int64_t)e * width;
-    float sum = 0.f;
-    for (int d = lane; d < width; d += 64) sum = fmaf(to_float<T>(row[d]), w_row[d], sum);
-    sum = wave_sum(sum);
+    const float sum = wave_sum(router_dot<T>(row, w + (int64_t)e * width, width, lane));
     if (lane == 0) s_score[e] = sum;
   }
   __syncthreads();
@@ -183,6 +205,7 @@ __global__ __launch_bounds__(256) void moe_route_wave_kernel(
       open = ahead < keep;
     }
   }
+  const int cols = top + options.fixed;
   int slot = -1;       // which of the token's choices this lane's expert is
   for (int j = 0; j < top; ++j) {
     const float offer = open ? choice : -INFINITY;
@@ -192,13 +215,17 @@ __global__ __launch_bounds__(256) void moe_route_wave_kernel(
     if (lane == chosen) {
       open = false;
       slot = j;
-      if (wave == 0) ids[t * top + j] = chosen;
+      if (wave == 0) ids[t * cols + j] = chosen;
     }
   }
   const float own = (slot >= 0 && score == score) ? score : 0.f;
   const float chosen_sum = wave_sum(own);
   if (slot >= 0 && wave == 0) {
-    weights[t * top + slot] = options.normalise ? own / (chosen_sum + 1e-20f) * scale : own * scale;
+    weights[t * cols + slot] = options.normalise ? own / (chosen_sum + 1e-20f) * scale : own * scale;
+  }
+  if (wave == 1 && lane < options.fixed) {
+    ids[t * cols + top + lane] = experts + lane;
+    weights[t * cols + top + lane] = 1.0f;
   }
 }
 
@@ -218,11 +245,16 @@ __device__ inline float moe_activation(float g, float u) {
 template <typename T, int ROWS, bool GATED>
 __global__ __launch_bounds__(256) void moe_hidden_kernel(
     const T* __restrict__ x, int64_t x_ld, const T* __restrict__ w1, const int* __restrict__ ids,
-    T* __restrict__ hidden, int width, int inner) {
+    T* __restrict__ hidden, int width, int inner, int experts, const T* __restrict__ w1x) {
   extern __shared__ float s_x[];
   // (blockIdx.x: the token, blockIdx.z: which of its choices)
   const int64_t row_index = (int64_t)blockIdx.x * gridDim.z + blockIdx.z;
-  const int e = ids[row_index];
+  int e = ids[row_index];
+  // (experts numbered from `experts` on lie in a tensor of their own)
+  if (e >= experts) {
+    e = w1x != nullptr ? e - experts : 0;
+    if (w1x != nullptr) w1 = w1x;
+  }
   const T* x_row = x + (int64_t)blockIdx.x * x_ld;
   for (int d = threadIdx.x; d < width; d += 256) s_x[d] = to_float<T>(x_row[d]);
   __syncthreads();
@@ -250,7 +282,8 @@ __global__ __launch_bounds__(256) void moe_hidden_kernel(
 template <typename T, int ROWS>
 __global__ __launch_bounds__(256) void moe_down_kernel(
     const T* __restrict__ hidden, const T* __restrict__ w2, const int* __restrict__ ids,
-    const float* __restrict__ weights, float* __restrict__ y, int width, int inner, int top) {
+    const float* __restrict__ weights, float* __restrict__ y, int width, int inner, int top,
+    int experts, const T* __restrict__ w2x) {
   extern __shared__ float s_h[];        // [top][inner]
   const int64_t t = blockIdx.x;
   for (int i = threadIdx.x; i < top * inner; i += 256)
@@ -264,7 +297,9 @@ __global__ __launch_bounds__(256) void moe_down_kernel(
     float total = 0.f;
     for (int j = 0; j < top; ++j) {
       const int e = ids[t * top + j];
-      const T* w_row = w2 + ((int64_t)e * width + d) * inner;
+      const T* w_row = (e < experts || w2x == nullptr)
+                           ? w2 + ((int64_t)(e < experts ? e : 0) * width + d) * inner
+                           : w2x + ((int64_t)(e - experts) * width + d) * inner;
       float sum = 0.f;
       for (int c = lane; c < inner; c += 64) sum = fmaf(to_float<T>(w_row[c]), s_h[j * inner + c], sum);
       total = fmaf(weights[t * top + j], wave_sum(sum), total);
@@ -275,7 +310,7 @@ __global__ __launch_bounds__(256) void moe_down_kernel(
 
 extern "C" int ps_moe_route(const void* x, int64_t x_ld, const float* w, int tokens, int width,
                             int experts, int groups, int keep, int top, float scale, int sigmoid,
-                            const float* correction, int group_top, int normalise, int* ids,
+                            const float* correction, int group_top, int normalise, int fixed, int* ids,
                             float* weights, int dtype, void* stream) {
   PS_REQUIRE(tokens >= 0 && width > 0 && experts > 0 && experts <= MOE_MAX_EXPERTS,
              "ps_moe_route: %d experts, at most %d", experts, MOE_MAX_EXPERTS);
@@ -288,7 +323,8 @@ extern "C" int ps_moe_route(const void* x, int64_t x_ld, const float* w, int tok
              "ps_moe_route: a group's score sums its %d largest scores, 1 to 8 are taken", group_top);
   if (tokens == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
-  const RouteOptions options = {sigmoid, correction, group_top, normalise};
+  PS_REQUIRE(fixed >= 0 && fixed <= 64, "ps_moe_route: %d fixed experts, up to 64 are taken", fixed);
+  const RouteOptions options = {sigmoid, correction, group_top, normalise, fixed};
   if (experts <= 64) {
     if (dtype == PS_F32)
       hipLaunchKernelGGL(moe_route_wave_kernel<float>, dim3(tokens), dim3(256), 0, s, (const float*)x,
@@ -334,10 +370,14 @@ __device__ inline void load8<float>(const float* p, float (&v)[8]) {
 template <typename T, int ROWS, bool GATED>
 __global__ __launch_bounds__(256) void moe_hidden_wide_kernel(
     const T* __restrict__ x, int64_t x_ld, const T* __restrict__ w1, const int* __restrict__ ids,
-    T* __restrict__ hidden, int width, int inner) {
+    T* __restrict__ hidden, int width, int inner, int experts, const T* __restrict__ w1x) {
   extern __shared__ float s_x[];
   const int64_t row_index = (int64_t)blockIdx.x * gridDim.z + blockIdx.z;
-  const int e = ids[row_index];
+  int e = ids[row_index];
+  if (e >= experts) {
+    e = w1x != nullptr ? e - experts : 0;
+    if (w1x != nullptr) w1 = w1x;
+  }
   const T* x_row = x + (int64_t)blockIdx.x * x_ld;
   for (int d = threadIdx.x; d < width; d += 256) s_x[d] = to_float<T>(x_row[d]);
   __syncthreads();
@@ -382,7 +422,8 @@ __global__ __launch_bounds__(256) void moe_hidden_wide_kernel(
 template <typename T, int ROWS>
 __global__ __launch_bounds__(256) void moe_down_wide_kernel(
     const T* __restrict__ hidden, const T* __restrict__ w2, const int* __restrict__ ids,
-    const float* __restrict__ weights, float* __restrict__ y, int width, int inner, int top) {
+    const float* __restrict__ weights, float* __restrict__ y, int width, int inner, int top,
+    int experts, const T* __restrict__ w2x) {
   extern __shared__ float s_h[];        // [top][inner]
   const int64_t t = blockIdx.x;
   for (int i = threadIdx.x; i < top * inner; i += 256)
@@ -403,7 +444,8 @@ __global__ __launch_bounds__(256) void moe_down_wide_kernel(
     for (int r = 0; r < ROWS; ++r) {
       sum[r] = 0.f;
       const int d = first + r < width ? first + r : width - 1;
-      rows[r] = w2 + ((int64_t)e * width + d) * inner;
+      rows[r] = (e < experts || w2x == nullptr) ? w2 + ((int64_t)(e < experts ? e : 0) * width + d) * inner
+                                                : w2x + ((int64_t)(e - experts) * width + d) * inner;
     }
     for (int c = lane * 8; c < inner; c += 512) {
       float hv[8];
@@ -622,8 +664,8 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
 
 extern "C" int ps_moe_experts(const void* x, int64_t x_ld, const void* w1, const void* w2,
                               const int* ids, const float* weights, void* hidden, float* y,
-                              int tokens, int width, int inner, int top, int gated, int dtype,
-                              void* stream) {
+                              int tokens, int width, int inner, int top, int gated, int experts,
+                              const void* w1x, const void* w2x, int dtype, void* stream) {
   PS_REQUIRE(tokens >= 0 && width > 0 && inner > 0 && top > 0 && top <= 65535,
              "ps_moe_experts: bad sizes");
   PS_REQUIRE((size_t)width * 4 <= 64 * 1024 && (size_t)top * inner * 4 <= 64 * 1024,
@@ -641,10 +683,11 @@ extern "C" int ps_moe_experts(const void* x, int64_t x_ld, const void* w1, const
     if (wide1)                                                                                     \
       hipLaunchKernelGGL((moe_hidden_wide_kernel<T, ROWS, GATED>), grid1, dim3(256),               \
                          (size_t)width * 4, s, (const T*)x, x_ld, (const T*)w1, ids, (T*)hidden,   \
-                         width, inner);                                                            \
+                         width, inner, experts, (const T*)w1x);                                    \
     else                                                                                           \
       hipLaunchKernelGGL((moe_hidden_kernel<T, ROWS, GATED>), grid1, dim3(256), (size_t)width * 4, \
-                         s, (const T*)x, x_ld, (const T*)w1, ids, (T*)hidden, width, inner);       \
+                         s, (const T*)x, x_ld, (const T*)w1, ids, (T*)hidden, width, inner,        \
+                         experts, (const T*)w1x);                                                  \
   } while (0)
 #define PS_MOE_ROWS(T, ROWS)                                                                       \
   do {                                                                                             \
@@ -653,10 +696,12 @@ extern "C" int ps_moe_experts(const void* x, int64_t x_ld, const void* w1, const
     else PS_MOE_HIDDEN(T, ROWS, false);                                                            \
     if (wide2)                                                                                     \
       hipLaunchKernelGGL((moe_down_wide_kernel<T, ROWS>), grid2, dim3(256), (size_t)top * inner * 4, \
-                         s, (const T*)hidden, (const T*)w2, ids, weights, y, width, inner, top);   \
+                         s, (const T*)hidden, (const T*)w2, ids, weights, y, width, inner, top,    \
+                         experts, (const T*)w2x);                                                  \
     else                                                                                           \
       hipLaunchKernelGGL((moe_down_kernel<T, ROWS>), grid2, dim3(256), (size_t)top * inner * 4, s, \
-                         (const T*)hidden, (const T*)w2, ids, weights, y, width, inner, top);      \
+                         (const T*)hidden, (const T*)w2, ids, weights, y, width, inner, top,       \
+                         experts, (const T*)w2x);                                                  \
   } while (0)
   if (dtype == PS_F32) {
     if (few) PS_MOE_ROWS(float, 2);

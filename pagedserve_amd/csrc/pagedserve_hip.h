@@ -429,12 +429,14 @@ int ps_lru_scan(const float* proj, int64_t ld, int y_col, int x_col, const float
 // equal groups of neighbours, a group's score being its largest s).
 int ps_moe_route(const void* x, int64_t x_ld, const float* w, int tokens, int width, int experts,
                  int groups, int keep, int top, float scale, int sigmoid, const float* correction,
-                 int group_top, int normalise, int* ids, float* weights, int dtype, void* stream);
+                 int group_top, int normalise, int fixed, int* ids, float* weights, int dtype,
+                 void* stream);
 // y[t] += sum_j weights[t, j] W2[e] (silu(W1[e][:inner] x_t) * (W1[e][inner:] x_t)), e = ids[t, j];
 // w1: [experts, 2 * inner, width], w2: [experts, width, inner]; hidden: [tokens * top, inner] scratch.
 int ps_moe_experts(const void* x, int64_t x_ld, const void* w1, const void* w2, const int* ids,
                    const float* weights, void* hidden, float* y, int tokens, int width, int inner,
-                   int top, int gated, int dtype, void* stream);
+                   int top, int gated, int experts, const void* w1x, const void* w2x, int dtype,
+                   void* stream);
 // The same for many rows in bfloat16 (width and inner multiples of 8): the (token, choice) pairs
 // are sorted by expert into tiles of 128 and multiplied on the matrix cores.  order:
 // [tiles * 128] int and tile_expert: [tiles] int scratch with tiles = ps_moe_grouped_tiles(tokens *

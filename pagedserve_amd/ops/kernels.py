@@ -83,12 +83,12 @@ _SIGNATURES = {
     "ps_pair_norm_mix": [c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_float, c_void_p, c_int,
                          c_int, c_void_p],
     "ps_moe_route": [c_void_p, c_int64, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float,
-                     c_int, c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p],
+                     c_int, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p],
     "ps_moe_experts_grouped": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
                                c_int, c_void_p],
     "ps_moe_experts": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
-                       c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+                       c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p],
     "ps_gla_output": [c_void_p, c_void_p, c_float, c_void_p, c_int64, c_void_p, c_int64, c_int,
                       c_int, c_int, c_int, c_void_p],
     "ps_softcap": [c_void_p, c_int64, c_int, c_int, c_float, c_void_p],
@@ -1766,13 +1766,15 @@ def pair_norm_mix(a, b, weight_a, weight_b, eps, share, y, tokens, width):
 
 
 def moe_route(x, router, groups, keep, top, scale, ids, weights, sigmoid=False, correction=None,
-              group_top=1, normalise=False):
+              group_top=1, normalise=False, fixed=0):
     """The experts that every row of ``x`` chooses (``ids``, int32 ``[tokens, top]``) and their
     weights (float): softmax (or ``sigmoid``) over all experts of the 32-bit logits, group-limited
     choice, the scores times ``scale`` (``csrc/moe.hip``).  ``correction``: a float per expert
     that is added to the scores for the choice only; ``group_top``: a group's score is the sum of
     that many of its largest choice scores; ``normalise``: the chosen scores are divided by
-    their sum before ``scale``."""
+    their sum before ``scale``.  ``fixed``: that many more columns of ``ids`` and ``weights`` are
+    filled with the numbers ``experts, experts + 1, ..`` and the weight one (experts that every token
+    uses, for ``moe_experts(extra=...)``)."""
     if correction is not None:
         _float_vector(correction, "correction", router.shape[0])
     if not 1 <= int(group_top) <= 8:
@@ -1786,11 +1788,11 @@ def moe_route(x, router, groups, keep, top, scale, ids, weights, sigmoid=False, 
     _check(ids, "ids", torch.int32, 2)
     _check(weights, "weights", torch.float32, 2)
     for tensor in (ids, weights):
-        if tensor.shape[0] < tokens or tensor.shape[1] != top or not tensor.is_contiguous():
-            raise KernelError("moe_route: ids and weights must be contiguous [>= tokens, top]")
+        if tensor.shape[0] < tokens or tensor.shape[1] != top + fixed or not tensor.is_contiguous():
+            raise KernelError("moe_route: ids and weights must be contiguous [>= tokens, top + fixed]")
     _call("ps_moe_route", x.data_ptr(), x.stride(0), router.data_ptr(), tokens, width, experts,
           int(groups), int(keep), int(top), float(scale), 1 if sigmoid else 0, _ptr(correction),
-          int(group_top), 1 if normalise else 0, ids.data_ptr(), weights.data_ptr(),
+          int(group_top), 1 if normalise else 0, int(fixed), ids.data_ptr(), weights.data_ptr(),
           dtype_code(x.dtype), _stream())
 
 
@@ -1839,10 +1841,12 @@ def moe_experts_grouped(x, w1, w2, ids, weights, hidden, out, order, tile_expert
           y.data_ptr(), tokens, width, inner, experts, top, 1 if gated else 0, _stream())
 
 
-def moe_experts(x, w1, w2, ids, weights, hidden, y, gated=True):
+def moe_experts(x, w1, w2, ids, weights, hidden, y, gated=True, extra=None):
     """``y[t] += sum_j weights[t, j] W2[e] (silu(W1[e][:inner] x_t) * (W1[e][inner:] x_t))`` with
     ``e = ids[t, j]``; ``w1``: ``[experts, 2 * inner, width]``, ``w2``: ``[experts, width, inner]``.
-    ``gated=False``: the plain form ``W2[e] relu(W1[e] x_t)^2`` with ``w1 [experts, inner, width]``."""
+    ``gated=False``: the plain form ``W2[e] relu(W1[e] x_t)^2`` with ``w1 [experts, inner, width]``.
+    ``extra = (w1x, w2x)``: experts numbered from ``experts`` on, in tensors of their own of the same
+    form (``moe_route(fixed=...)`` names them for every token)."""
     _check(x, "x", ndim=2)
     tokens, width = x.shape
     _check(w1, "w1", x.dtype, 3)
@@ -1857,10 +1861,20 @@ def moe_experts(x, w1, w2, ids, weights, hidden, y, gated=True):
     _check(hidden, "hidden", x.dtype, 2)
     if hidden.shape[0] < tokens * top or hidden.shape[1] != inner or not hidden.is_contiguous():
         raise KernelError("moe_experts: hidden must be contiguous [>= tokens * top, inner]")
+    if not (ids.is_contiguous() and weights.is_contiguous()) or weights.shape[1] != top:
+        raise KernelError("moe_experts: ids and weights must be contiguous [tokens, top]")
+    w1x = w2x = None
+    if extra is not None:
+        w1x, w2x = extra
+        _check(w1x, "extra w1", x.dtype, 3)
+        _check(w2x, "extra w2", x.dtype, 3)
+        if (tuple(w1x.shape[1:]) != tuple(w1.shape[1:]) or tuple(w2x.shape[1:]) != tuple(w2.shape[1:])
+                or w1x.shape[0] != w2x.shape[0] or not (w1x.is_contiguous() and w2x.is_contiguous())):
+            raise KernelError("moe_experts: the extra experts must have the form of the others")
     _float_rows(y, "y", tokens, width)
     _call("ps_moe_experts", x.data_ptr(), x.stride(0), w1.data_ptr(), w2.data_ptr(), ids.data_ptr(),
           weights.data_ptr(), hidden.data_ptr(), y.data_ptr(), tokens, width, inner, top,
-          1 if gated else 0, dtype_code(x.dtype), _stream())
+          1 if gated else 0, experts, _ptr(w1x), _ptr(w2x), dtype_code(x.dtype), _stream())
 
 
 def gla_output(o, weight, eps, gate, out, heads, value_dim):

@@ -128,7 +128,10 @@ class MixtureOfExperts(FeedForward):
     ``normalise``: the chosen scores are divided by their sum (+ 1e-20) before ``scale``;
     ``form="relu2"``: an expert is ``W_down,e relu(W_up,e x)^2`` (``up.weight [experts * inner,
     width]``); ``shared_inner > 0``: one more expert of the same form and that inner width
-    (``shared.*``) runs for every token with weight one."""
+    (``shared.*``) runs for every token with weight one.  Steps of few tokens run a shared
+    expert of the plain form whose inner width is a multiple of the others' inside the experts'
+    own two launches, cut into experts of their width that every token uses (squaring is element
+    by element, so the cut is exact); steps of many tokens run it as two dense products."""
 
     graph_safe = True
 
@@ -169,11 +172,16 @@ class MixtureOfExperts(FeedForward):
         self.first_rows = (2 if self.gated else 1) * inner     # rows of an expert's first matrix
         self.first_name = "gate_up.weight" if self.gated else "up.weight"
         self.shared = None
+        self.shared_pieces = 0      # the shared expert as that many experts of the others' width
         if shared_inner:
             if self.gated:
                 self.shared = GatedFeedForward(width, dtype, shared_inner)
             else:
                 self.shared = DenseFeedForward(width, dtype, shared_inner, "relu2", bias=False)
+                pieces = shared_inner // inner
+                # (the row kernels keep a token's hidden rows of all its experts in LDS)
+                if shared_inner == pieces * inner and pieces <= 64 and (top + pieces) * inner * 4 <= 64 * 1024:
+                    self.shared_pieces = pieces
 
     def parameters(self):
         params = {
@@ -197,19 +205,28 @@ class MixtureOfExperts(FeedForward):
         self.down_weight = tensors["down.weight"].view(self.experts, self.width, self.inner)
         if self.shared is not None:
             self.shared.bind({name: tensors["shared." + name] for name in self.shared.parameters()})
+        if self.shared_pieces:
+            pieces = self.shared_pieces
+            self.shared_extra = (
+                self.shared.up_weight.view(pieces, self.inner, self.width),
+                self.shared.down_weight.view(self.width, pieces, self.inner).transpose(0, 1).contiguous())
 
     def forward(self, x, residual, ctx):
         tokens = ctx.tokens
         workspace = ctx.workspace
-        ids = workspace.first_rows("moe_ids", self.top, torch.int32, tokens)
-        weights = workspace.first_rows("moe_weights", self.top, torch.float32, tokens)
+        sorted_path = (tokens * self.top >= kernels.MOE_GROUPED_FROM
+                       and kernels.moe_grouped_supported(self.dtype, self.width, self.inner))
+        # few tokens: the shared expert's pieces ride along as experts that every token uses
+        fixed = 0 if sorted_path else self.shared_pieces
+        chosen = self.top + fixed
+        ids = workspace.first_rows("moe_ids", chosen, torch.int32, tokens)
+        weights = workspace.first_rows("moe_weights", chosen, torch.float32, tokens)
         kernels.moe_route(x, self.router_weight, self.groups, self.keep, self.top, self.scale, ids,
                           weights, sigmoid=self.sigmoid, correction=self.correction,
-                          group_top=self.group_top, normalise=self.normalise)
-        most = workspace.max_rows * self.top
+                          group_top=self.group_top, normalise=self.normalise, fixed=fixed)
+        most = workspace.max_rows * (self.top + self.shared_pieces)
         hidden = workspace.rows("moe_hidden", self.inner, self.dtype, max_rows=most)
-        if (tokens * self.top >= kernels.MOE_GROUPED_FROM
-                and kernels.moe_grouped_supported(self.dtype, self.width, self.inner)):
+        if sorted_path:
             # many rows: sorted by expert, tiles on the matrix cores
             tiles = kernels.moe_grouped_tiles(most, self.experts)
             kernels.moe_experts_grouped(
@@ -219,6 +236,6 @@ class MixtureOfExperts(FeedForward):
                 workspace.flat("moe_tiles", tiles, torch.int32), residual, gated=self.gated)
         else:
             kernels.moe_experts(x, self.first_weight, self.down_weight, ids, weights, hidden, residual,
-                                gated=self.gated)
-        if self.shared is not None:
+                                gated=self.gated, extra=self.shared_extra if fixed else None)
+        if self.shared is not None and not fixed:
             self.shared.forward(x, residual, ctx)

@@ -240,6 +240,45 @@ def test_squared_relu_experts_by_rows_and_sorted_onto_the_matrix_cores(dtype, wi
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("width,inner,experts,top,pieces", [(48, 20, 5, 2, 2), (128, 64, 8, 3, 1), (44, 24, 70, 2, 3)])
+def test_a_shared_expert_cut_into_experts_that_every_token_uses(dtype, width, inner, experts, top, pieces):
+    """The router names the pieces behind its own choices with the weight one, and the row
+    kernels find them in tensors of their own: the sum is the routed experts' plus one dense
+    squared-ReLU expert of ``pieces * inner`` hidden columns."""
+    kernels = _kernels()
+    g = torch.Generator().manual_seed(width + experts)
+    tokens = 6
+    x = torch.randn((tokens, width), generator=g).to(dtype)
+    router = torch.randn((experts, width), generator=g) * 0.5
+    correction = torch.randn(experts, generator=g) * 0.2
+    w1 = (torch.randn((experts, inner, width), generator=g) / width ** 0.5).to(dtype)
+    w2 = (torch.randn((experts, width, inner), generator=g) / inner ** 0.5).to(dtype)
+    shared_up = (torch.randn((pieces * inner, width), generator=g) / width ** 0.5).to(dtype)
+    shared_down = (torch.randn((width, pieces * inner), generator=g) / inner ** 0.5).to(dtype)
+    spec = {"experts": experts, "top": top, "scale": 1.3, "groups": {"count": 1, "keep": 1}}
+    chosen, weights = plain.route(x.double(), {"r.router": router.double(), "r.correction": correction.double()}, "r.", spec)
+    ids = torch.full((tokens, top + pieces), -1, dtype=torch.int32, device="cuda")
+    got = torch.zeros((tokens, top + pieces), device="cuda")
+    kernels.moe_route(x.cuda(), router.cuda(), 1, 1, top, 1.3, ids, got, sigmoid=True, correction=correction.cuda(),
+                      group_top=2, normalise=True, fixed=pieces)
+    assert ids[:, top:].cpu().tolist() == [list(range(experts, experts + pieces))] * tokens
+    assert torch.equal(got[:, top:].cpu(), torch.ones(tokens, pieces))
+    assert [sorted(row) for row in ids[:, :top].cpu().tolist()] == [sorted(row) for row in chosen]
+    y0 = torch.randn((tokens, width), generator=g)
+    expected = y0.double() + plain.relu2(x.double() @ shared_up.double().T) @ shared_down.double().T
+    for t in range(tokens):
+        for e, weight in zip(chosen[t], weights[t].tolist()):
+            expected[t] += weight * (plain.relu2(x[t].double() @ w1[e].double().T) @ w2[e].double().T)
+    extra = (shared_up.cuda().view(pieces, inner, width),
+             shared_down.cuda().view(width, pieces, inner).transpose(0, 1).contiguous())
+    y = y0.clone().cuda()
+    hidden = torch.empty((tokens * (top + pieces), inner), dtype=dtype, device="cuda")
+    kernels.moe_experts(x.cuda(), w1.cuda(), w2.cuda(), ids, got, hidden, y, gated=False, extra=extra)
+    tol = 1e-4 if dtype == torch.float32 else 4e-2
+    assert torch.allclose(y.double().cpu(), expected, atol=tol, rtol=tol)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_gate_with_the_tanh_form_of_gelu(dtype):
     kernels = _kernels()
     g = torch.Generator().manual_seed(2)
