@@ -642,3 +642,42 @@ def test_drawn_configurations_in_mixed_batches(tmp_path, seed, dtype):
         good, what = _close(rows, reference, dtype)
         assert good, (seed, name, what, raw)
         engine.cache.check_invariants()
+
+
+def test_the_trace_program_replays_a_mixed_trace(tmp_path):
+    """``bin/trace_run`` as a user calls it, on a Kozapel folder: JSON lines in, ``<step>.f32``
+    files and ``done`` lines out, a pool made for the live requests only."""
+    import json
+    import os
+    import subprocess
+    import sys
+
+    import numpy as np
+
+    folder, raw, tensors, _ = kozapel_models.folder_of(tmp_path, "C")
+    requests = _requests(raw, (70, 1, 23, 40, 9), 31)
+    reference = _reference(raw, tensors, requests)
+    steps = helpers.trace_mixed(requests, max_live=4, seed=3)
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out_dir = tmp_path / "out"
+    process = subprocess.run(
+        [sys.executable, os.path.join(root, "bin", "trace_run"), "--model", folder, "--dtype", "float32",
+         "--out", str(out_dir), "--max-tokens", str(helpers.live_token_budget(steps))],
+        input="\n".join(json.dumps(step) for step in steps) + "\n", capture_output=True, text=True, timeout=600)
+    assert process.returncode == 0, process.stderr[-2000:]
+    done = [line for line in process.stdout.splitlines() if line.startswith("done ")]
+    assert done == [f"done {step['step']}" for step in steps]
+    held, rows = {}, {}
+    for step in steps:
+        wanted = sum(len(entry["want"]) for entry in step["entries"])
+        values = np.fromfile(out_dir / f"{step['step']}.f32", dtype="<f4").reshape(wanted, raw["vocab"])
+        row = 0
+        for entry in step["entries"]:
+            start = held.get(entry["id"], 0)
+            for place in entry["want"]:
+                rows[(entry["id"], start + place)] = torch.from_numpy(values[row]).double()
+                row += 1
+            held[entry["id"]] = start + len(entry["tokens"])
+    worst, scale, where = helpers.max_error(rows, reference)
+    assert len(rows) == sum(len(tokens) for tokens in requests.values())
+    assert worst <= TOLERANCE["float32"] * scale, (worst / scale, where)
