@@ -1,6 +1,6 @@
 from . import (attention, block, connection, differential_attention, embedding, feed_forward,  # noqa: F401
-               latent_attention,
-               linear_attention, norm, position, side_by_side, state_space)  # noqa: F401  (register kinds)
+               latent_attention, linear_attention, norm, position, side_by_side,  # noqa: F401
+               state_space)  # noqa: F401  (register kinds)
 from .base import (CacheView, Embedding, FeedForward, Head, Mixer, Norm, PagedKVSpec, Part,
                    PositionEncoding, SlotStateSpec, StepContext, StepItem, Workspace)
 from .registry import (ARRANGEMENTS, CONNECTIONS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS, POSITIONS, ROLES,
