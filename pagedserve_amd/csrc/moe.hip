@@ -459,12 +459,16 @@ __global__ __launch_bounds__(256) void moe_down_wide_kernel(
         for (int i = 0; i < 8; ++i) sum[r] = fmaf(a[i], hv[i], sum[r]);
       }
     }
+    // (a lane's share of all experts is summed first and the lanes meet once at the end: no
+    // expert's loads wait for the one before)
 #pragma unroll
-    for (int r = 0; r < ROWS; ++r) total[r] = fmaf(weight, wave_sum(sum[r]), total[r]);
+    for (int r = 0; r < ROWS; ++r) total[r] = fmaf(weight, sum[r], total[r]);
   }
 #pragma unroll
-  for (int r = 0; r < ROWS; ++r)
-    if (lane == 0 && first + r < width) y[t * width + first + r] += total[r];
+  for (int r = 0; r < ROWS; ++r) {
+    const float whole = wave_sum(total[r]);
+    if (lane == 0 && first + r < width) y[t * width + first + r] += whole;
+  }
 }
 
 // ---- many rows: the (token, choice) pairs sorted by expert, products on the matrix cores -------
