@@ -110,13 +110,16 @@ __global__ __launch_bounds__(256) void gemm_nt_tiled_kernel(
     const int row = load_row + i * 64;
     a_row_ok[i] = m0 + row < m;
     w_row_ok[i] = n0 + row < n;
-    a_src[i] = a + (int64_t)(a_row_ok[i] ? m0 + row : 0) * lda + load_k;
-    w_src[i] = w + (int64_t)(w_row_ok[i] ? n0 + row : 0) * k + load_k;
+    a_src[i] = a + (int64_t)(a_row_ok[i] ? m0 + row : 0) * lda;
+    w_src[i] = w + (int64_t)(w_row_ok[i] ? n0 + row : 0) * k;
   }
   auto load_global = [&](uint4* stage_a, uint4* stage_w, int k0) {
-    // unconditional loads from clamped addresses, zeroed afterwards
+    // unconditional loads from clamped addresses, zeroed afterwards.  The stand-in for a chunk
+    // behind the range's end is the range's own first chunk: this thread's chunk of the first k
+    // tile lies behind the row's end where the range is shorter than a tile (k under 32), and
+    // for a matrix's last row behind the matrix
     const bool k_ok = k0 + load_k < k_end;
-    const int kk = k_ok ? k0 : k_begin;
+    const int kk = k_ok ? k0 + load_k : k_begin;
     const uint4 zero = {0u, 0u, 0u, 0u};
 #pragma unroll
     for (int i = 0; i < 2; ++i) {

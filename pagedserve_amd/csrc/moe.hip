@@ -549,20 +549,23 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
   for (int i = 0; i < 2; ++i) {
     const int a_pair = s_pair[a_row + i * 64];
     a_ok[i] = a_pair >= 0;
-    a_src[i] = a + (int64_t)(a_pair < 0 ? 0 : (FROM_TOKENS ? a_pair / top : a_pair)) * lda + chunk;
+    a_src[i] = a + (int64_t)(a_pair < 0 ? 0 : (FROM_TOKENS ? a_pair / top : a_pair)) * lda;
     const int local = a_row + i * 64;      // 0..127
     int row;
     if (HIDDEN) row = (local < 64 ? 0 : columns) + n0 + (local & 63);
     else row = n0 + local;
     w_ok[i] = HIDDEN ? n0 + (local & 63) < columns : ((MODE == 2 || local < 64) && row < w_rows);
-    w_src[i] = w + (int64_t)e * expert_stride + (int64_t)(w_ok[i] ? row : 0) * k + chunk;
+    w_src[i] = w + (int64_t)e * expert_stride + (int64_t)(w_ok[i] ? row : 0) * k;
   }
   // a ring of MOE_DEPTH stages in registers keeps that many k tiles' loads in flight
   uint4 ring_a[MOE_DEPTH][2], ring_w[MOE_DEPTH][2];
   const uint4 zero = {0u, 0u, 0u, 0u};
   auto load_global = [&](uint4* stage_a, uint4* stage_w, int k0) {
+    // (a chunk behind the row's end is not read at all: the row's own first chunk stands in for
+    // it and is thrown away; with k under 32 the old stand-in, this chunk of the first k tile, lay
+    // behind the end of the row, and for the last row of the last expert behind the tensor)
     const bool k_ok = k0 + chunk < k;
-    const int kk = k_ok ? k0 : 0;
+    const int kk = k_ok ? k0 + chunk : 0;
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       stage_a[i] = *reinterpret_cast<const uint4*>(a_src[i] + kk);

@@ -206,7 +206,8 @@ def test_sigmoid_router_with_corrections_groups_by_their_two_best_and_normed_wei
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("width,inner,experts,top,tokens", [(48, 20, 5, 2, 19), (128, 96, 4, 3, 7), (44, 24, 5, 2, 3),
-                                                            (64, 40, 5, 2, 150), (72, 136, 7, 1, 333)])
+                                                            (64, 40, 5, 2, 150), (72, 136, 7, 1, 333),
+                                                            (24, 16, 3, 2, 100), (200, 8, 2, 2, 70)])
 def test_squared_relu_experts_by_rows_and_sorted_onto_the_matrix_cores(dtype, width, inner, experts, top, tokens):
     kernels = _kernels()
     g = torch.Generator().manual_seed(width + inner)
@@ -681,3 +682,35 @@ def test_the_trace_program_replays_a_mixed_trace(tmp_path):
     worst, scale, where = helpers.max_error(rows, reference)
     assert len(rows) == sum(len(tokens) for tokens in requests.values())
     assert worst <= TOLERANCE["float32"] * scale, (worst / scale, where)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("seed", range(30, 44))
+def test_drawn_configurations_with_long_prompts(tmp_path, seed, dtype):
+    """More drawn configurations under prompts of a few hundred tokens, whole and in long
+    portions beside decoded tokens of four live requests: the tiled attention kernels over windows
+    of a few tokens, experts sorted onto the matrix cores at inner widths under one k tile (whose
+    stand-in loads once reached behind the last expert's last row), a prompt of 70 tokens and then
+    decoding."""
+    import os
+
+    raw, page_size = _drawn_configuration(seed)
+    folder = os.path.join(str(tmp_path), f"drawn_{seed}")
+    weights = plain.random_checkpoint(raw, 100 + seed)
+    if dtype == "bfloat16":
+        for name in weights:      # (no close calls: see above)
+            if name.endswith("mlp.correction"):
+                order = torch.randperm(weights[name].numel(), generator=torch.Generator().manual_seed(seed))
+                weights[name] = order.float() * 3.0
+    tensors = kozapel_models.write_folder(folder, raw, weights)
+    requests = _requests(raw, (230, 130, 64, 3, 1), 7 + seed)
+    reference = _reference(raw, tensors, requests)
+    for name, steps in (("mixed", helpers.trace_mixed(requests, max_live=4, portion=(70, 2, 150, 9),
+                                                      decode_tail=12, seed=seed)),
+                        ("whole", helpers.trace_whole(requests)),
+                        ("decoded", helpers.trace_tail_decoded({"r1": requests["r1"]}, tail=60))):
+        engine = _engine(folder, dtype, page_size, steps, max_requests=4)
+        rows = helpers.replay_in_process(engine, steps)
+        good, what = _close(rows, reference, dtype)
+        assert good, (seed, name, what, raw)
+        engine.cache.check_invariants()
