@@ -3,8 +3,6 @@ or kernel option alone, then small models of several shapes stepped whole, decod
 token, in portions down to two tokens, and in mixed batches whose pages and slots are used again;
 a key that stands out just inside and just outside a window, and far back through a latent."""
 
-import math
-
 import pytest
 import torch
 
