@@ -712,3 +712,26 @@ def test_drawn_configurations_with_long_prompts(tmp_path, seed, dtype):
         good, what = _close(rows, reference, dtype)
         assert good, (seed, name, what, raw)
         engine.cache.check_invariants()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_sixteen_requests_decoding_together_over_long_contexts(tmp_path, dtype):
+    """Sixteen requests of two heads (four maps) decode side by side over 150 to 200 keys without
+    a window: a (token, head) pair per quarter compute unit, where the split-KV kernel runs blocks
+    of sixteen waves, here leaving records that the merge of both maps reads."""
+    folder, raw, tensors, page_size = kozapel_models.folder_of(tmp_path, "D")
+    requests = _requests(raw, tuple(150 + 3 * index for index in range(16)), 71)
+    reference = _reference(raw, tensors, requests)
+    tail = 6
+    steps = [{"step": index, "entries": [{"id": rid, "tokens": tokens[:-tail], "want": [len(tokens) - tail - 1]}],
+              "end": []} for index, (rid, tokens) in enumerate(requests.items())]
+    for back in range(tail, 0, -1):
+        steps.append({"step": len(steps), "entries": [{"id": rid, "tokens": [tokens[-back]], "want": [0]}
+                                                      for rid, tokens in requests.items()], "end": []})
+    steps[-1]["end"] = list(requests)
+    engine = _engine(folder, dtype, page_size, steps, max_requests=16)
+    rows = helpers.replay_in_process(engine, steps)
+    assert len(rows) == 16 * (tail + 1)
+    good, what = _close(rows, reference, dtype)
+    assert good, what
+    engine.cache.check_invariants()
