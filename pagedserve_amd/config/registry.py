@@ -37,6 +37,9 @@ class Architecture:
     presets: tuple = ()      # ((name, raw config dict), ...)
     # (config, name -> stored shape) -> config: sizes that only the checkpoint's tensors give
     complete_config: Callable[[Any, Callable], Any] = None
+    # (raw config dict, name -> stored shape or None) -> raw config dict: sizes that the file
+    # leaves out and the tensors' shapes give, filled in before the typed configuration is read
+    complete_raw: Callable[[dict, Callable], dict] = None
 
 
 ARCHITECTURES: Dict[str, Architecture] = {}

@@ -151,6 +151,71 @@ def weight_sources(config: KozapelConfig, spec: ModelSpec):
     return sources
 
 
+def complete_raw(raw: dict, shape_of) -> dict:
+    """The raw configuration with the sizes that it leaves out filled in from the shapes of the
+    stored tensors (``shape_of(name)``: the shape, or None where the file has no such tensor).  A
+    size that the file names is never touched; one that no tensor gives stays out, and the typed
+    reader then reports it."""
+    import copy
+
+    raw = copy.deepcopy(raw)
+
+    def rows(name, axis=0):
+        shape = shape_of(name)
+        return None if shape is None or len(shape) <= axis else int(shape[axis])
+
+    def fill(target, key, value):
+        if isinstance(target, dict) and key not in target and value is not None and value > 0:
+            target[key] = int(value)
+
+    def ratio(a, b):
+        return a // b if a is not None and b and a % b == 0 else None
+
+    fill(raw, "vocab", rows("embed"))
+    fill(raw, "width", rows("embed", 1))
+    fill(raw, "streams", rows("l0.hc1.in"))
+    listed = raw.get("layers")
+    if not isinstance(listed, list):
+        return raw
+    for index, layer in enumerate(listed):
+        if not isinstance(layer, dict) or not isinstance(layer.get("mixer"), dict):
+            continue
+        m, p = layer["mixer"], f"l{index}.mix."
+        if layer.get("type") == "attention":
+            fill(m, "dim", rows(p + "lq1"))
+            dim = m.get("dim")
+            fill(m, "heads", ratio(rows(p + "q"), 2 * dim if dim else 0))
+            source = m.get("kv_from")
+            if source is None:
+                fill(m, "kv_heads", ratio(rows(p + "k"), 2 * dim if dim else 0))
+                fill(m, "vdim", ratio(rows(p + "v"), m.get("kv_heads")))
+            else:
+                fill(m, "vdim", ratio(rows(p + "o", 1), m.get("heads")))
+                if isinstance(source, int) and 0 <= source < index and isinstance(listed[source].get("mixer"), dict):
+                    fill(m, "kv_heads", listed[source]["mixer"].get("kv_heads"))
+        elif layer.get("type") == "latent_attention":
+            fill(m, "q_rank", rows(p + "dq"))
+            fill(m, "kv_rank", rows(p + "dkv.norm"))
+            if m.get("kv_rank") and rows(p + "dkv") is not None and "rot_dim" not in m:
+                m["rot_dim"] = rows(p + "dkv") - m["kv_rank"]
+            if "heads" not in m and m.get("rot_dim") and rows(p + "uq") is not None and rows(p + "uk") is not None:
+                fill(m, "heads", ratio(rows(p + "uq") - rows(p + "uk"), m["rot_dim"]))
+            fill(m, "dim", ratio(rows(p + "uk"), m.get("heads")))
+            fill(m, "vdim", ratio(rows(p + "uv"), m.get("heads")))
+        mlp, f = layer.get("mlp"), f"l{index}.mlp."
+        if isinstance(mlp, dict):
+            if mlp.get("kind", "dense") == "dense":
+                fill(mlp, "ff", rows(f + "gate"))
+            else:
+                if rows(f + "e0.up") is not None:
+                    fill(mlp.setdefault("expert", {}), "ff", rows(f + "e0.up"))
+                if isinstance(mlp.get("router"), dict):
+                    fill(mlp["router"], "experts", rows(f + "router"))
+                if rows(f + "shared.up") is not None:
+                    fill(mlp.setdefault("shared", {}), "ff", rows(f + "shared.up"))
+    return raw
+
+
 def random_tensors(config: KozapelConfig, seed: int, device="cpu"):
     """Checkpoint tensors of a random model, drawn from one seeded generator in a fixed order.
     Matrices N(0, 1/sqrt(in)); scales, corrections and the stream weights such that every part
@@ -222,5 +287,6 @@ KOZAPEL = register_architecture(Architecture(
     build_spec=build_spec,
     weight_sources=weight_sources,
     random_tensors=random_tensors,
+    complete_raw=complete_raw,
     model_type="kozapel",
 ))

@@ -28,6 +28,11 @@ def load_model(folder, dtype="float32", device="cuda"):
     """(model, typed config) of the folder's ``config.json`` + ``model.safetensors``."""
     raw = read_config_json(folder)
     architecture = resolve_architecture(raw)
+    if architecture.complete_raw is not None:
+        with SafetensorsFile(os.path.join(folder, "model.safetensors")) as handle:
+            stored = canonical_names(handle.names(), architecture.strip_prefixes)
+            raw = architecture.complete_raw(
+                raw, lambda name: tuple(handle.shape(stored[name])) if name in stored else None)
     config = architecture.config_class.from_dict(raw)
     if architecture.complete_config is not None:
         with SafetensorsFile(os.path.join(folder, "model.safetensors")) as handle:

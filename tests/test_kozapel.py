@@ -231,3 +231,40 @@ def test_the_router_keeps_the_best_groups_and_norms_the_weights():
     w["r.correction"][4:] = -9.5
     chosen, _ = plain.route(h, w, "r.", router)
     assert chosen[0] == [0, 1]
+
+
+@pytest.mark.parametrize("which", sorted(kozapel_models.MODELS))
+def test_sizes_that_the_file_leaves_out_come_from_the_tensors(tmp_path, which):
+    """Every size that a tensor's shape gives may be missing from ``config.json``: the loader
+    fills it in before the typed configuration is read, and names what still lacks."""
+    import json
+
+    folder, raw, tensors, _ = kozapel_models.folder_of(tmp_path, which)
+    full, _ = load_model(folder, dtype="float32", device="cpu")
+    stripped = copy.deepcopy(raw)
+    for key in ("vocab", "width", "streams"):
+        stripped.pop(key, None)
+    for layer in stripped["layers"]:
+        for key in ("dim", "vdim", "kv_heads", "q_rank", "kv_rank", "rot_dim"):
+            layer["mixer"].pop(key, None)
+        if layer["type"] == "attention" or layer["mixer"].get("rot"):
+            layer["mixer"].pop("heads", None)
+        mlp = layer["mlp"]
+        if mlp is not None and mlp["kind"] == "dense":
+            mlp.pop("ff")
+        elif mlp is not None:
+            mlp.pop("expert")
+            mlp["router"].pop("experts")
+            mlp.pop("shared", None)
+    with open(folder + "/config.json", "w") as handle:
+        json.dump(stripped, handle)
+    again, config = load_model(folder, dtype="float32", device="cpu")
+    assert config == KozapelConfig.from_dict(raw)
+    assert again.parameter_count == full.parameter_count
+    # a size that no tensor gives is still reported by its name
+    del stripped["layers"][0]["mixer"]["scale"]
+    with open(folder + "/config.json", "w") as handle:
+        json.dump(stripped, handle)
+    with pytest.raises(ConfigError) as caught:
+        load_model(folder, dtype="float32", device="cpu")
+    assert "scale" in str(caught.value)
